@@ -1,0 +1,181 @@
+/*
+ * quick_ssm_hip.h -- C ABI of libquick_ssm_hip.so, the gfx950 (MI355X) implementation of
+ * quick_ssm's gated linear scan
+ *
+ *     h(t) = a(t) * h(t-1) + b(t) * x(t),   h(-1) = 0
+ *     y(t) = c(t) * h(t)
+ *
+ * and of its reverse-time gradient
+ *
+ *     dH(t) = c(t) * dy(t) + a(t+1) * dH(t+1),   dH(L) = 0
+ *     dx = b * dH,  db = x * dH,  da(t) = h(t-1) * dH(t),  dc = dy * h.
+ *
+ * The reference has no native layer (its device code is six Triton kernels launched from
+ * Python), so the entry points below are what a binding of its device path would call.  Each
+ * one names the reference function it stands in for.
+ *
+ * Conventions
+ *   - All tensors are [B, L, D] with D contiguous (element stride 1).  Batch and time strides
+ *     are passed in elements, so sliced views need no copy.
+ *   - Plain pointers and sizes only; every buffer is owned by the caller.  The library never
+ *     allocates device memory and never synchronises: kernels are enqueued on `stream`.
+ *   - Arithmetic is fp32 whatever the storage type; y and the gradients are rounded once.
+ *   - Return value: 0 on success, a QSSM_E* code or a hipError_t (> 0) otherwise;
+ *     qssm_error_string() describes the last failure on the calling thread.
+ *   - Entry points are re-entrant.  Two launches that share one workspace must be ordered
+ *     on one stream.
+ */
+#ifndef QUICK_SSM_HIP_H
+#define QUICK_SSM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(__GNUC__)
+#define QSSM_API __attribute__((visibility("default")))
+#else
+#define QSSM_API
+#endif
+
+#define QSSM_VERSION 100 /* major*10000 + minor*100 + patch */
+
+/* storage types */
+#define QSSM_F32 0
+#define QSSM_F16 1
+#define QSSM_BF16 2
+
+/* error codes (negative; positive values are hipError_t) */
+#define QSSM_EINVAL (-1)    /* bad argument (null pointer, size, dtype, plan mismatch) */
+#define QSSM_EALIGN (-2)    /* pointer or stride not aligned to plan.vec elements */
+#define QSSM_EWORKSPACE (-3)/* workspace smaller than plan.workspace_bytes */
+#define QSSM_ESTATE (-4)    /* device status word reports a failed launch */
+
+/* plan directions */
+#define QSSM_FORWARD 0
+#define QSSM_BACKWARD 1
+
+/*
+ * Launch geometry of one scan launch.  A "tile" is one workgroup's share: a strip of
+ * `strip_cols` adjacent columns of one batch row, times `seg_len` consecutive time steps.
+ * Tiles of one (batch, strip) chain hand a one-row carry to the next tile in time through the
+ * workspace; `ckpt_stride` is the spacing of the fp32 states h(t-1) kept for the backward.
+ */
+typedef struct qssm_plan {
+  int32_t B, L, D;
+  int32_t in_dtype;       /* x, a, b, c and dx, da, db, dc */
+  int32_t out_dtype;      /* y and dy */
+  int32_t direction;      /* QSSM_FORWARD / QSSM_BACKWARD */
+  int32_t vec;            /* adjacent columns per lane: 1, 2 or 4 */
+  int32_t steps;          /* consecutive time steps per lane: 4 or 8 */
+  int32_t g_log2;         /* log2(lanes per row of a strip) */
+  int32_t strip_cols;     /* vec << g_log2 */
+  int32_t seg_len;        /* steps * (256 >> g_log2) */
+  int32_t n_strips;       /* ceil(D / strip_cols) */
+  int32_t n_seg;          /* ceil(L / seg_len) */
+  int32_t ckpt_stride;    /* spacing (time steps) of saved states; divides seg_len */
+  int32_t n_ckpt;         /* ceil(L / ckpt_stride) */
+  int32_t reserved;
+  uint64_t workspace_bytes; /* carry workspace the launch needs (zero-filled, see below) */
+  uint64_t ckpt_elems;      /* B * n_ckpt * D floats */
+} qssm_plan;
+
+/* element strides of one [B, L, D] tensor; the D stride is 1 by contract */
+typedef struct qssm_strides {
+  int64_t b, l;
+} qssm_strides;
+
+/* Library version (QSSM_VERSION of the build). */
+QSSM_API int qssm_version(void);
+
+/* Text for the last error raised on the calling thread ("" if none). */
+QSSM_API const char* qssm_error_string(void);
+
+/*
+ * Choose the launch geometry for a shape.
+ *   align_elems : largest power of two (<= 4) that divides D, every batch/time stride, and
+ *                 every base address expressed in elements, over all tensors of the launch.
+ *   ckpt_stride : 0 lets the forward plan pick; a backward plan (and a forward plan that must
+ *                 match one) passes the stride the saved states were written with.
+ *   tune        : 0 = automatic; otherwise (g_log2 + 1) | (steps << 8) overrides for sweeps.
+ * Stands in for the grid/block arithmetic of block_scan_forward_3d
+ * (quick_ssm/triton_forwards.py:157-167) and block_scan_backward_3d
+ * (quick_ssm/triton_backwards.py:195-204).
+ */
+QSSM_API int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int32_t out_dtype,
+                   int32_t direction, int32_t align_elems, int32_t ckpt_stride, int32_t tune,
+                   qssm_plan* plan);
+
+/*
+ * Zero-fill a carry workspace (a fill kernel on `stream`, safe under graph capture).  A
+ * workspace must be zero before its first launch; each launch leaves it zero again, so this is
+ * needed once per allocation and after a launch that reported QSSM_ESTATE.
+ */
+QSSM_API int qssm_workspace_reset(void* workspace, uint64_t bytes, void* stream);
+
+/*
+ * Read back the status word of a workspace (synchronises `stream`).  0 = every launch since
+ * the last reset completed; nonzero = a tile gave up waiting for its neighbour's carry and
+ * the outputs of that launch are poisoned with NaN.
+ */
+QSSM_API int qssm_workspace_status(const void* workspace, void* stream, int32_t* status);
+
+/*
+ * Forward scan: one pass that reads x, a, b, c once and writes y once.
+ *   c          may be NULL (treated as 1, so y = h): the block_scan_forward_3d case.
+ *   y          may be NULL (state-only pass: only `ckpt` is produced).
+ *   h_out      optional fp32 [B, L, D] (strides sh): every h(t); the checkpoint=False case.
+ *   ckpt       optional fp32 [B, n_ckpt, D] contiguous: h(t-1) at t = k * ckpt_stride.
+ * Replaces _TritonScanFunction.forward's per-tile body (quick_ssm/scan_interface.py:91-107):
+ * block_scan_forward_3d (quick_ssm/triton_forwards.py:134-172, three launches + fp32 scratch)
+ * followed by y = c * h and the cast to out_dtype.
+ */
+QSSM_API int qssm_scan_forward(const qssm_plan* plan,
+                      const void* x, qssm_strides sx,
+                      const void* a, qssm_strides sa,
+                      const void* b, qssm_strides sb,
+                      const void* c, qssm_strides sc,
+                      void* y, qssm_strides sy,
+                      float* h_out, qssm_strides sh,
+                      float* ckpt,
+                      void* workspace, uint64_t workspace_bytes,
+                      void* stream);
+
+/*
+ * Backward scan: one reverse-time pass that reads x, a, b, c, dy once and writes dx, da, db,
+ * dc once.  h is rebuilt inside each tile from `ckpt` (the checkpoint=True case), or read from
+ * `h` when that is given (the checkpoint=False case and block_scan_backward_3d's signature);
+ * exactly one of `ckpt` / `h` must be non-NULL.  Any of dx, da, db, dc may be NULL (skipped).
+ * Replaces _TritonScanFunction.backward's per-tile body (quick_ssm/scan_interface.py:125-145):
+ * the forward re-run (:133-134) plus block_scan_backward_3d
+ * (quick_ssm/triton_backwards.py:168-209) plus the casts at :148-152.
+ */
+QSSM_API int qssm_scan_backward(const qssm_plan* plan,
+                       const void* x, qssm_strides sx,
+                       const void* a, qssm_strides sa,
+                       const void* b, qssm_strides sb,
+                       const void* c, qssm_strides sc,
+                       const void* dy, qssm_strides sdy,
+                       const float* h, qssm_strides sh,
+                       const float* ckpt,
+                       void* dx, qssm_strides sdx,
+                       void* da, qssm_strides sda,
+                       void* db, qssm_strides sdb,
+                       void* dc, qssm_strides sdc,
+                       void* workspace, uint64_t workspace_bytes,
+                       void* stream);
+
+/*
+ * Streaming copy of `bytes` bytes (16-byte aligned, multiple of 16) on `stream`.  Not part of
+ * the scan: it is the known-size kernel against which rocprof's FETCH_SIZE / WRITE_SIZE
+ * counters and the achievable-bandwidth ceiling are calibrated by the benchmark.
+ */
+QSSM_API int qssm_copy_bytes(void* dst, const void* src, uint64_t bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QUICK_SSM_HIP_H */

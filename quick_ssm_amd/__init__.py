@@ -1,0 +1,9 @@
+"""quick_ssm on MI355X: the gated linear scan as hand-written HIP kernels for gfx950.
+
+Public surface is the reference's (quick_ssm/__init__.py:1-4): `scan`, `SSM`, `RMSNorm`.
+"""
+from .scan_interface import scan
+from .layers import SSM, RMSNorm
+
+__all__ = ["scan", "SSM", "RMSNorm"]
+__version__ = "0.1.0"

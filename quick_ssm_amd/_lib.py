@@ -1,0 +1,127 @@
+"""ctypes binding of libquick_ssm_hip.so (the C ABI declared in include/quick_ssm_hip.h).
+
+The library is looked up next to this file.  It is never replaced by another implementation:
+if it cannot be loaded, every device entry point raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from pathlib import Path
+from typing import Optional
+
+LIB_NAME = "libquick_ssm_hip.so"
+LIB_PATH = Path(__file__).resolve().parent / LIB_NAME
+
+QSSM_F32, QSSM_F16, QSSM_BF16 = 0, 1, 2
+QSSM_FORWARD, QSSM_BACKWARD = 0, 1
+QSSM_EINVAL, QSSM_EALIGN, QSSM_EWORKSPACE, QSSM_ESTATE = -1, -2, -3, -4
+
+EXPORTED_SYMBOLS = (
+    "qssm_version",
+    "qssm_error_string",
+    "qssm_plan_scan",
+    "qssm_workspace_reset",
+    "qssm_workspace_status",
+    "qssm_scan_forward",
+    "qssm_scan_backward",
+    "qssm_copy_bytes",
+)
+
+
+class Plan(ctypes.Structure):
+    """Mirror of `qssm_plan`."""
+
+    _fields_ = [
+        ("B", ctypes.c_int32),
+        ("L", ctypes.c_int32),
+        ("D", ctypes.c_int32),
+        ("in_dtype", ctypes.c_int32),
+        ("out_dtype", ctypes.c_int32),
+        ("direction", ctypes.c_int32),
+        ("vec", ctypes.c_int32),
+        ("steps", ctypes.c_int32),
+        ("g_log2", ctypes.c_int32),
+        ("strip_cols", ctypes.c_int32),
+        ("seg_len", ctypes.c_int32),
+        ("n_strips", ctypes.c_int32),
+        ("n_seg", ctypes.c_int32),
+        ("ckpt_stride", ctypes.c_int32),
+        ("n_ckpt", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+        ("workspace_bytes", ctypes.c_uint64),
+        ("ckpt_elems", ctypes.c_uint64),
+    ]
+
+    def describe(self) -> dict:
+        return {name: int(getattr(self, name)) for name, _ in self._fields_ if name != "reserved"}
+
+
+class Strides(ctypes.Structure):
+    """Mirror of `qssm_strides` (element strides of the batch and time axes)."""
+
+    _fields_ = [("b", ctypes.c_int64), ("l", ctypes.c_int64)]
+
+
+class QssmError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(f"libquick_ssm_hip: {message} (code {code})")
+        self.code = code
+
+
+_lock = threading.Lock()
+_lib: Optional[ctypes.CDLL] = None
+
+
+def _declare(lib: ctypes.CDLL) -> None:
+    vp, u64, i32 = ctypes.c_void_p, ctypes.c_uint64, ctypes.c_int32
+    lib.qssm_version.restype = ctypes.c_int
+    lib.qssm_version.argtypes = []
+    lib.qssm_error_string.restype = ctypes.c_char_p
+    lib.qssm_error_string.argtypes = []
+    lib.qssm_plan_scan.restype = ctypes.c_int
+    lib.qssm_plan_scan.argtypes = [i32] * 9 + [ctypes.POINTER(Plan)]
+    lib.qssm_workspace_reset.restype = ctypes.c_int
+    lib.qssm_workspace_reset.argtypes = [vp, u64, vp]
+    lib.qssm_workspace_status.restype = ctypes.c_int
+    lib.qssm_workspace_status.argtypes = [vp, vp, ctypes.POINTER(i32)]
+    lib.qssm_scan_forward.restype = ctypes.c_int
+    lib.qssm_scan_forward.argtypes = (
+        [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, u64, vp]
+    )
+    lib.qssm_scan_backward.restype = ctypes.c_int
+    lib.qssm_scan_backward.argtypes = (
+        [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, Strides] * 4 + [vp, u64, vp]
+    )
+    lib.qssm_copy_bytes.restype = ctypes.c_int
+    lib.qssm_copy_bytes.argtypes = [vp, vp, u64, vp]
+
+
+def is_built() -> bool:
+    return LIB_PATH.exists()
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library (once).  Raises RuntimeError if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is None:
+            if not LIB_PATH.exists():
+                raise RuntimeError(
+                    f"{LIB_PATH} is missing: the HIP scan kernels are not built. "
+                    "Run `python -m quick_ssm_amd.build` (needs hipcc). There is no other device path."
+                )
+            lib = ctypes.CDLL(os.fspath(LIB_PATH))
+            _declare(lib)
+            _lib = lib
+    return _lib
+
+
+def check(code: int) -> None:
+    """Raise QssmError for a nonzero return code of a library call."""
+    if code != 0:
+        message = load().qssm_error_string().decode("utf-8", "replace")
+        raise QssmError(code, message or "call failed")

@@ -1,0 +1,313 @@
+// C ABI of libquick_ssm_hip.so: launch planning, argument checks and kernel launches.
+// Declarations and the reference functions each entry point stands in for: include/quick_ssm_hip.h.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "scan_common.h"
+
+namespace qssm {
+
+static thread_local char g_err[256] = "";
+
+static int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+static int hip_fail(hipError_t e, const char* what) {
+  snprintf(g_err, sizeof(g_err), "%s: %s", what, hipGetErrorString(e));
+  return (int)e;
+}
+
+static int dtype_size(int dt) {
+  switch (dt) {
+    case QSSM_F32: return 4;
+    case QSSM_F16: return 2;
+    case QSSM_BF16: return 2;
+    default: return 0;
+  }
+}
+
+static int pow2_ceil(int64_t n) {
+  int p = 1;
+  while (p < n) p <<= 1;
+  return p;
+}
+
+// Lanes that one row of D columns can feed at `vec` columns per lane (a power of two <= 256).
+static int lanes_cap(int D, int vec) {
+  const int lanes = pow2_ceil(D > 0 ? (D + vec - 1) / vec : 1);
+  return lanes < kThreads ? lanes : kThreads;
+}
+
+static int ilog2(int n) {
+  int l = 0;
+  while ((1 << l) < n) ++l;
+  return l;
+}
+
+__global__ void __launch_bounds__(256) fill_zero_kernel(uint4* p, uint64_t n16) {
+  uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (; i < n16; i += stride) p[i] = make_uint4(0, 0, 0, 0);
+}
+
+// Grid-stride 16-byte copy: the calibration kernel of known traffic (bytes read = bytes written).
+__global__ void __launch_bounds__(256) copy_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src,
+                                                   uint64_t n16) {
+  uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (; i + 3 * stride < n16; i += 4 * stride) {
+    const uint4 v0 = src[i], v1 = src[i + stride], v2 = src[i + 2 * stride], v3 = src[i + 3 * stride];
+    dst[i] = v0;
+    dst[i + stride] = v1;
+    dst[i + 2 * stride] = v2;
+    dst[i + 3 * stride] = v3;
+  }
+  for (; i < n16; i += stride) dst[i] = src[i];
+}
+
+static bool aligned_to(const void* p, int64_t sb, int64_t sl, int elem_bytes, int vec) {
+  if (p == nullptr) return true;
+  if (((uintptr_t)p) % ((uintptr_t)elem_bytes * vec) != 0) return false;
+  return (sb % vec == 0) && (sl % vec == 0);
+}
+
+static int check_plan(const qssm_plan* pl, int direction) {
+  if (pl == nullptr) return fail(QSSM_EINVAL, "plan is NULL");
+  if (pl->direction != direction) return fail(QSSM_EINVAL, "plan was made for the other direction");
+  if (pl->B < 0 || pl->L < 0 || pl->D < 0) return fail(QSSM_EINVAL, "negative dimension");
+  if (pl->vec != 1 && pl->vec != 2 && pl->vec != 4) return fail(QSSM_EINVAL, "plan.vec must be 1, 2 or 4");
+  if (pl->steps != 4 && pl->steps != 8) return fail(QSSM_EINVAL, "plan.steps must be 4 or 8");
+  if (pl->g_log2 < 0 || pl->g_log2 > 8) return fail(QSSM_EINVAL, "plan.g_log2 out of range");
+  if (pl->D % pl->vec != 0) return fail(QSSM_EALIGN, "D=%d is not a multiple of plan.vec=%d", pl->D, pl->vec);
+  const int ng = kThreads >> pl->g_log2;
+  if (pl->strip_cols != (pl->vec << pl->g_log2) || pl->seg_len != pl->steps * ng)
+    return fail(QSSM_EINVAL, "plan geometry is inconsistent");
+  if (pl->B == 0 || pl->L == 0 || pl->D == 0) return 0;
+  if (pl->n_strips != (pl->D + pl->strip_cols - 1) / pl->strip_cols ||
+      pl->n_seg != (pl->L + pl->seg_len - 1) / pl->seg_len)
+    return fail(QSSM_EINVAL, "plan tile counts are inconsistent");
+  // Forward lanes write a saved state only at their own first step; backward tiles read one
+  // only at the tile's first step.
+  if (pl->ckpt_stride <= 0 || pl->seg_len % pl->ckpt_stride != 0 ||
+      (direction == QSSM_FORWARD && pl->ckpt_stride % pl->steps != 0) ||
+      pl->n_ckpt != (pl->L + pl->ckpt_stride - 1) / pl->ckpt_stride)
+    return fail(QSSM_EINVAL, "plan.ckpt_stride=%d does not fit seg_len=%d / steps=%d", pl->ckpt_stride,
+                pl->seg_len, pl->steps);
+  return 0;
+}
+
+static void fill_geometry(Geometry* g, const qssm_plan* pl, void* workspace) {
+  g->B = pl->B;
+  g->L = pl->L;
+  g->D = pl->D;
+  g->g_log2 = pl->g_log2;
+  g->n_strips = pl->n_strips;
+  g->n_chains = pl->B * pl->n_strips;
+  g->n_seg = pl->n_seg;
+  g->seg_len = pl->seg_len;
+  g->ckpt_stride = pl->ckpt_stride;
+  g->n_ckpt = pl->n_ckpt;
+  char* ws = (char*)workspace;
+  g->status = (int*)ws;
+  g->tickets = (unsigned*)(ws + kStatusBytes);
+  g->carry = (unsigned long long*)(ws + ws_carry_offset((uint64_t)g->n_chains));
+}
+
+}  // namespace qssm
+
+using namespace qssm;
+
+extern "C" {
+
+int qssm_version(void) { return QSSM_VERSION; }
+
+const char* qssm_error_string(void) { return g_err; }
+
+int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int32_t out_dtype, int32_t direction,
+                   int32_t align_elems, int32_t ckpt_stride, int32_t tune, qssm_plan* plan) {
+  if (plan == nullptr) return fail(QSSM_EINVAL, "plan is NULL");
+  if (B < 0 || L < 0 || D < 0) return fail(QSSM_EINVAL, "negative dimension");
+  if (direction != QSSM_FORWARD && direction != QSSM_BACKWARD) return fail(QSSM_EINVAL, "bad direction");
+  const int es = dtype_size(in_dtype), os = dtype_size(out_dtype);
+  if (es == 0 || os == 0) return fail(QSSM_EINVAL, "unknown dtype code");
+  if (direction == QSSM_FORWARD ? find_fwd_launcher(in_dtype, out_dtype) == nullptr
+                                : find_bwd_launcher(in_dtype, out_dtype) == nullptr)
+    return fail(QSSM_EINVAL, "dtype pair (in=%d, out=%d) is not built; cast on the host", in_dtype, out_dtype);
+  if (align_elems < 1) align_elems = 1;
+
+  memset(plan, 0, sizeof(*plan));
+  plan->B = B;
+  plan->L = L;
+  plan->D = D;
+  plan->in_dtype = in_dtype;
+  plan->out_dtype = out_dtype;
+  plan->direction = direction;
+
+  // Widest lane vector the alignment allows: 8 bytes per lane for 16-bit storage, 16 for fp32
+  // forward; the backward keeps 5 operands + h in registers, so fp32 stays at 8 bytes there.
+  int vec = 4;
+  if (es == 4 && direction == QSSM_BACKWARD) vec = 2;
+  while (vec > 1 && (align_elems % vec != 0 || (D > 0 && D % vec != 0))) vec >>= 1;
+  plan->vec = vec;
+
+  // Steps per lane: 8 keeps chains short; the backward at 8 bytes per lane would not fit the
+  // register file at 8 steps.
+  int steps = 8;
+  if (direction == QSSM_BACKWARD && vec * es >= 8) steps = 4;
+
+  // Lanes per row: 128-byte row pieces when D allows, never more lanes than the row has vectors.
+  const int cap = lanes_cap(D, vec);
+  int g = 128 / (vec * es);
+  if (g < 1) g = 1;
+  if (tune != 0) {
+    const int tg = (tune & 0xff) - 1, ts = (tune >> 8) & 0xff;
+    if (tg >= 0 && tg <= 8) g = 1 << tg;
+    if (ts == 4 || ts == 8) steps = ts;
+  } else {
+    // Short sequences: widen the rows rather than leave most time groups idle.
+    const int64_t lp2 = pow2_ceil(L > 0 ? L : 1);
+    while (g < cap && (int64_t)steps * (kThreads / g) / 2 >= lp2) g <<= 1;
+  }
+  if (g > cap) g = cap;
+  if (ckpt_stride > 0) {
+    // A tile must cover a whole number of saved-state intervals and a lane must not straddle one.
+    if ((ckpt_stride & (ckpt_stride - 1)) != 0 || ckpt_stride < 4)
+      return fail(QSSM_EINVAL, "ckpt_stride=%d must be a power of two >= 4", ckpt_stride);
+    if (direction == QSSM_FORWARD && ckpt_stride % steps != 0) steps = 4;
+    while (steps * (kThreads / g) < ckpt_stride && g > 1) g >>= 1;
+    if ((steps * (kThreads / g)) % ckpt_stride != 0)
+      return fail(QSSM_EINVAL, "ckpt_stride=%d does not fit any tile length", ckpt_stride);
+  }
+  plan->steps = steps;
+  plan->g_log2 = ilog2(g);
+  plan->strip_cols = vec << plan->g_log2;
+  plan->seg_len = steps * (kThreads >> plan->g_log2);
+  if (ckpt_stride > 0 && plan->seg_len % ckpt_stride != 0)
+    return fail(QSSM_EINVAL, "ckpt_stride=%d does not divide seg_len=%d", ckpt_stride, plan->seg_len);
+  plan->ckpt_stride = ckpt_stride > 0 ? ckpt_stride : plan->seg_len;
+  if (B == 0 || L == 0 || D == 0) return 0;
+  plan->n_strips = (D + plan->strip_cols - 1) / plan->strip_cols;
+  plan->n_seg = (L + plan->seg_len - 1) / plan->seg_len;
+  plan->n_ckpt = (L + plan->ckpt_stride - 1) / plan->ckpt_stride;
+  const uint64_t n_chains = (uint64_t)B * plan->n_strips;
+  if (n_chains * plan->n_seg > 0x7fffffffull) return fail(QSSM_EINVAL, "shape needs more than 2^31 tiles");
+  plan->workspace_bytes =
+      ws_carry_offset(n_chains) + (plan->n_seg > 1 ? n_chains * plan->n_seg * plan->strip_cols * 8ull : 0ull);
+  plan->ckpt_elems = (uint64_t)B * plan->n_ckpt * D;
+  return 0;
+}
+
+int qssm_workspace_reset(void* workspace, uint64_t bytes, void* stream) {
+  if (workspace == nullptr || bytes == 0) return 0;
+  if (((uintptr_t)workspace) % 16 != 0 || bytes % 16 != 0)
+    return fail(QSSM_EALIGN, "workspace must be 16-byte aligned and a multiple of 16 bytes");
+  const uint64_t n16 = bytes / 16;
+  uint64_t blocks = (n16 + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (uint4*)workspace,
+                     n16);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : hip_fail(e, "fill_zero_kernel launch");
+}
+
+int qssm_workspace_status(const void* workspace, void* stream, int32_t* status) {
+  if (workspace == nullptr || status == nullptr) return fail(QSSM_EINVAL, "NULL argument");
+  hipError_t e = hipMemcpyAsync(status, workspace, sizeof(int32_t), hipMemcpyDeviceToHost, (hipStream_t)stream);
+  if (e != hipSuccess) return hip_fail(e, "hipMemcpyAsync(status)");
+  e = hipStreamSynchronize((hipStream_t)stream);
+  return e == hipSuccess ? 0 : hip_fail(e, "hipStreamSynchronize");
+}
+
+int qssm_scan_forward(const qssm_plan* plan, const void* x, qssm_strides sx, const void* a, qssm_strides sa,
+                      const void* b, qssm_strides sb, const void* c, qssm_strides sc, void* y, qssm_strides sy,
+                      float* h_out, qssm_strides sh, float* ckpt, void* workspace, uint64_t workspace_bytes,
+                      void* stream) {
+  int rc = check_plan(plan, QSSM_FORWARD);
+  if (rc != 0) return rc;
+  if (plan->B == 0 || plan->L == 0 || plan->D == 0) return 0;
+  if (x == nullptr || a == nullptr || b == nullptr) return fail(QSSM_EINVAL, "x, a, b must not be NULL");
+  if (y == nullptr && h_out == nullptr && ckpt == nullptr) return fail(QSSM_EINVAL, "no output requested");
+  fwd_launch_fn fn = find_fwd_launcher(plan->in_dtype, plan->out_dtype);
+  if (fn == nullptr) return fail(QSSM_EINVAL, "dtype pair is not built");
+  const int es = dtype_size(plan->in_dtype), os = dtype_size(plan->out_dtype), v = plan->vec;
+  if (!aligned_to(x, sx.b, sx.l, es, v) || !aligned_to(a, sa.b, sa.l, es, v) || !aligned_to(b, sb.b, sb.l, es, v) ||
+      !aligned_to(c, sc.b, sc.l, es, v) || !aligned_to(y, sy.b, sy.l, os, v) ||
+      !aligned_to(h_out, sh.b, sh.l, 4, v) || !aligned_to(ckpt, 0, 0, 4, v))
+    return fail(QSSM_EALIGN, "a pointer or stride is not aligned to plan.vec=%d elements", v);
+  if (workspace == nullptr || workspace_bytes < plan->workspace_bytes)
+    return fail(QSSM_EWORKSPACE, "workspace has %llu bytes, plan needs %llu", (unsigned long long)workspace_bytes,
+                (unsigned long long)plan->workspace_bytes);
+
+  FwdArgs args;
+  fill_geometry(&args.g, plan, workspace);
+  args.x = x; args.a = a; args.b = b; args.c = c; args.y = y; args.h_out = h_out; args.ckpt = ckpt;
+  args.x_sb = sx.b; args.x_sl = sx.l; args.a_sb = sa.b; args.a_sl = sa.l;
+  args.b_sb = sb.b; args.b_sl = sb.l; args.c_sb = sc.b; args.c_sl = sc.l;
+  args.y_sb = sy.b; args.y_sl = sy.l; args.h_sb = sh.b; args.h_sl = sh.l;
+  const dim3 grid((unsigned)((uint64_t)args.g.n_chains * args.g.n_seg));
+  fn(args, plan->vec, plan->steps, grid, (hipStream_t)stream);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : hip_fail(e, "scan_fwd_kernel launch");
+}
+
+int qssm_scan_backward(const qssm_plan* plan, const void* x, qssm_strides sx, const void* a, qssm_strides sa,
+                       const void* b, qssm_strides sb, const void* c, qssm_strides sc, const void* dy,
+                       qssm_strides sdy, const float* h, qssm_strides sh, const float* ckpt, void* dx,
+                       qssm_strides sdx, void* da, qssm_strides sda, void* db, qssm_strides sdb, void* dc,
+                       qssm_strides sdc, void* workspace, uint64_t workspace_bytes, void* stream) {
+  int rc = check_plan(plan, QSSM_BACKWARD);
+  if (rc != 0) return rc;
+  if (plan->B == 0 || plan->L == 0 || plan->D == 0) return 0;
+  if (x == nullptr || a == nullptr || b == nullptr || c == nullptr || dy == nullptr)
+    return fail(QSSM_EINVAL, "x, a, b, c, dy must not be NULL");
+  if ((h == nullptr) == (ckpt == nullptr)) return fail(QSSM_EINVAL, "pass exactly one of h and ckpt");
+  bwd_launch_fn fn = find_bwd_launcher(plan->in_dtype, plan->out_dtype);
+  if (fn == nullptr) return fail(QSSM_EINVAL, "dtype pair is not built");
+  const int es = dtype_size(plan->in_dtype), os = dtype_size(plan->out_dtype), v = plan->vec;
+  if (!aligned_to(x, sx.b, sx.l, es, v) || !aligned_to(a, sa.b, sa.l, es, v) || !aligned_to(b, sb.b, sb.l, es, v) ||
+      !aligned_to(c, sc.b, sc.l, es, v) || !aligned_to(dy, sdy.b, sdy.l, os, v) ||
+      !aligned_to(h, sh.b, sh.l, 4, v) || !aligned_to(ckpt, 0, 0, 4, v) || !aligned_to(dx, sdx.b, sdx.l, es, v) ||
+      !aligned_to(da, sda.b, sda.l, es, v) || !aligned_to(db, sdb.b, sdb.l, es, v) ||
+      !aligned_to(dc, sdc.b, sdc.l, es, v))
+    return fail(QSSM_EALIGN, "a pointer or stride is not aligned to plan.vec=%d elements", v);
+  if (workspace == nullptr || workspace_bytes < plan->workspace_bytes)
+    return fail(QSSM_EWORKSPACE, "workspace has %llu bytes, plan needs %llu", (unsigned long long)workspace_bytes,
+                (unsigned long long)plan->workspace_bytes);
+
+  BwdArgs args;
+  fill_geometry(&args.g, plan, workspace);
+  args.x = x; args.a = a; args.b = b; args.c = c; args.dy = dy; args.h = h; args.ckpt = ckpt;
+  args.dx = dx; args.da = da; args.db = db; args.dc = dc;
+  args.x_sb = sx.b; args.x_sl = sx.l; args.a_sb = sa.b; args.a_sl = sa.l;
+  args.b_sb = sb.b; args.b_sl = sb.l; args.c_sb = sc.b; args.c_sl = sc.l;
+  args.dy_sb = sdy.b; args.dy_sl = sdy.l; args.h_sb = sh.b; args.h_sl = sh.l;
+  args.dx_sb = sdx.b; args.dx_sl = sdx.l; args.da_sb = sda.b; args.da_sl = sda.l;
+  args.db_sb = sdb.b; args.db_sl = sdb.l; args.dc_sb = sdc.b; args.dc_sl = sdc.l;
+  const dim3 grid((unsigned)((uint64_t)args.g.n_chains * args.g.n_seg));
+  fn(args, plan->vec, plan->steps, grid, (hipStream_t)stream);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : hip_fail(e, "scan_bwd_kernel launch");
+}
+
+int qssm_copy_bytes(void* dst, const void* src, uint64_t bytes, void* stream) {
+  if (bytes == 0) return 0;
+  if (dst == nullptr || src == nullptr) return fail(QSSM_EINVAL, "NULL argument");
+  if (((uintptr_t)dst) % 16 != 0 || ((uintptr_t)src) % 16 != 0 || bytes % 16 != 0)
+    return fail(QSSM_EALIGN, "copy needs 16-byte alignment and a multiple of 16 bytes");
+  const uint64_t n16 = bytes / 16;
+  uint64_t blocks = (n16 + 256 * 4 - 1) / (256 * 4);
+  if (blocks > 256 * 32) blocks = 256 * 32;
+  if (blocks == 0) blocks = 1;
+  hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (uint4*)dst,
+                     (const uint4*)src, n16);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : hip_fail(e, "copy_kernel launch");
+}
+
+}  // extern "C"

@@ -1,0 +1,275 @@
+"""Host side of the HIP scan: tensor checks, launch planning, workspace, and the two launches.
+
+Everything here is plumbing around `qssm_scan_forward` / `qssm_scan_backward`
+(include/quick_ssm_hip.h).  It takes the place of the launch code in the reference's
+`block_scan_forward_3d` (quick_ssm/triton_forwards.py:134-172) and `block_scan_backward_3d`
+(quick_ssm/triton_backwards.py:168-209): no fp32 upcast copies, no N-sized scratch, one launch per
+direction.
+"""
+from __future__ import annotations
+
+import ctypes
+import threading
+from typing import Dict, Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import Plan, Strides
+
+Tensor = torch.Tensor
+
+_DTYPE_CODE = {torch.float32: _lib.QSSM_F32, torch.float16: _lib.QSSM_F16, torch.bfloat16: _lib.QSSM_BF16}
+# (storage of x,a,b,c) -> storages of y the kernels are built for
+_BUILT_OUT = {
+    torch.float32: (torch.float32,),
+    torch.float16: (torch.float16, torch.float32),
+    torch.bfloat16: (torch.bfloat16, torch.float32),
+}
+
+_ws_lock = threading.Lock()
+_workspaces: Dict[Tuple[int, int], Tensor] = {}
+
+
+def kernel_dtypes(in_dtypes: Sequence[torch.dtype], out_dtype: torch.dtype) -> Tuple[torch.dtype, torch.dtype]:
+    """Storage types the launch will use for (x,a,b,c / grads) and for (y / dy).
+
+    Arithmetic is fp32 in every case.  Operands of mixed or unsupported storage are cast to a
+    common supported one on the host; an unsupported y storage is produced as fp32 and cast.
+    """
+    common = in_dtypes[0]
+    for dt in in_dtypes[1:]:
+        common = torch.promote_types(common, dt)
+    if common not in _DTYPE_CODE:
+        common = torch.float32
+    k_out = out_dtype if out_dtype in _BUILT_OUT[common] else torch.float32
+    return common, k_out
+
+
+def _unit_inner(t: Tensor) -> Tensor:
+    """A view or copy of `t` whose last axis is contiguous."""
+    if t.size(-1) > 1 and t.stride(-1) != 1:
+        return t.contiguous()
+    if t.size(-1) == 1 and t.stride(-1) != 1:
+        return t.contiguous()
+    return t
+
+
+def _strides(t: Optional[Tensor]) -> Strides:
+    if t is None:
+        return Strides(0, 0)
+    return Strides(t.stride(0), t.stride(1))
+
+
+def _ptr(t: Optional[Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _align_elems(tensors: Sequence[Optional[Tensor]], D: int) -> int:
+    """Largest v in (4, 2, 1) such that D, every stride and every base address (in elements) divide by v."""
+    for v in (4, 2):
+        ok = D % v == 0
+        for t in tensors:
+            if not ok:
+                break
+            if t is None:
+                continue
+            es = t.element_size()
+            ok = t.data_ptr() % (es * v) == 0 and t.stride(0) % v == 0 and t.stride(1) % v == 0
+        if ok:
+            return v
+    return 1
+
+
+def _workspace(device: torch.device, stream: int, nbytes: int) -> Tensor:
+    """Zero-initialised carry workspace for (device, stream), grown on demand.
+
+    A launch leaves its workspace zero again, so the buffer is filled once, at allocation
+    (torch.zeros runs a fill kernel on the current stream, ahead of the launch that uses it).
+    """
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
+    with _ws_lock:
+        ws = _workspaces.get(key)
+        if ws is None or ws.numel() < nbytes:
+            size = max(1 << 20, 1 << (int(nbytes) - 1).bit_length())
+            ws = torch.zeros(size, dtype=torch.uint8, device=device)
+            _workspaces[key] = ws
+        return ws
+
+
+def workspace_status(device: Optional[torch.device] = None) -> int:
+    """Status word of the current stream's workspace (synchronises).  0 = all launches completed."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else device
+    stream = torch.cuda.current_stream(device).cuda_stream
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
+    with _ws_lock:
+        ws = _workspaces.get(key)
+    if ws is None:
+        return 0
+    out = ctypes.c_int32(0)
+    _lib.check(_lib.load().qssm_workspace_status(ws.data_ptr(), stream, ctypes.byref(out)))
+    return int(out.value)
+
+
+def reset_workspaces() -> None:
+    """Drop every cached workspace (the next launch allocates a fresh zeroed one)."""
+    with _ws_lock:
+        _workspaces.clear()
+
+
+def make_plan(B: int, L: int, D: int, in_dtype: torch.dtype, out_dtype: torch.dtype, direction: int,
+              align_elems: int, ckpt_stride: int = 0, tune: int = 0) -> Plan:
+    plan = Plan()
+    _lib.check(
+        _lib.load().qssm_plan_scan(B, L, D, _DTYPE_CODE[in_dtype], _DTYPE_CODE[out_dtype], direction,
+                                   align_elems, ckpt_stride, tune, ctypes.byref(plan))
+    )
+    return plan
+
+
+def _require_gpu(*tensors: Tensor) -> torch.device:
+    dev = tensors[0].device
+    for t in tensors:
+        if t.device.type != "cuda":
+            raise RuntimeError("HIP scan backend requires GPU tensors.")
+        if t.device != dev:
+            raise RuntimeError("all scan operands must live on one GPU")
+    return dev
+
+
+def scan_forward(
+    x: Tensor, a: Tensor, b: Tensor, c: Optional[Tensor], *,
+    out_dtype: torch.dtype,
+    want_y: bool = True,
+    want_h: bool = False,
+    want_ckpt: bool = True,
+    tune: int = 0,
+    bwd_tune: int = 0,
+) -> Tuple[Optional[Tensor], Optional[Tensor], Optional[Tensor], int]:
+    """One forward launch.  Operands must already share one supported storage type.
+
+    Returns (y, h, ckpt, ckpt_stride): y in `out_dtype` (a storage the kernels are built for), h
+    the full fp32 state if `want_h`, ckpt the fp32 states h(t-1) at t = k*ckpt_stride if
+    `want_ckpt` (what the backward rebuilds h from).
+    """
+    ops = [x, a, b] + ([c] if c is not None else [])
+    dev = _require_gpu(*ops)
+    B, L, D = x.shape
+    in_dtype = x.dtype
+    y = torch.empty((B, L, D), dtype=out_dtype, device=dev) if want_y else None
+    h = torch.empty((B, L, D), dtype=torch.float32, device=dev) if want_h else None
+    if B == 0 or L == 0 or D == 0:
+        return y, h, (torch.empty((B, 0, D), dtype=torch.float32, device=dev) if want_ckpt else None), 0
+
+    x, a, b = _unit_inner(x), _unit_inner(a), _unit_inner(b)
+    c = _unit_inner(c) if c is not None else None
+    align = _align_elems([x, a, b, c, y, h], D)
+
+    ckpt_stride = 0
+    if want_ckpt:
+        # The backward decides how far apart the saved states may be; the forward follows.
+        ckpt_stride = make_plan(B, L, D, in_dtype, out_dtype, _lib.QSSM_BACKWARD, align, 0, bwd_tune).seg_len
+    plan = make_plan(B, L, D, in_dtype, out_dtype, _lib.QSSM_FORWARD, align, ckpt_stride, tune)
+    ckpt = None
+    if want_ckpt:
+        ckpt = torch.empty((B, plan.n_ckpt, D), dtype=torch.float32, device=dev)
+
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        ws = _workspace(dev, stream, int(plan.workspace_bytes))
+        _lib.check(
+            _lib.load().qssm_scan_forward(
+                ctypes.byref(plan),
+                _ptr(x), _strides(x), _ptr(a), _strides(a), _ptr(b), _strides(b), _ptr(c), _strides(c),
+                _ptr(y), _strides(y), _ptr(h), _strides(h), _ptr(ckpt),
+                ws.data_ptr(), ws.numel(), stream,
+            )
+        )
+    return y, h, ckpt, int(plan.ckpt_stride)
+
+
+def scan_backward(
+    x: Tensor, a: Tensor, b: Tensor, c: Tensor, dy: Tensor, *,
+    h: Optional[Tensor] = None,
+    ckpt: Optional[Tensor] = None,
+    ckpt_stride: int = 0,
+    need: Sequence[bool] = (True, True, True, True),
+    tune: int = 0,
+) -> Tuple[Optional[Tensor], Optional[Tensor], Optional[Tensor], Optional[Tensor]]:
+    """One backward launch.  x, a, b, c share one storage type; dy has the storage of y.
+
+    Exactly one of `h` (full fp32 state) and `ckpt` (+ its `ckpt_stride`) must be given.  Returns
+    (dx, da, db, dc) in the storage type of the operands; entries not in `need` are None.
+    """
+    dev = _require_gpu(x, a, b, c, dy)
+    B, L, D = x.shape
+    in_dtype = x.dtype
+    grads = [torch.empty((B, L, D), dtype=in_dtype, device=dev) if n else None for n in need]
+    if B == 0 or L == 0 or D == 0:
+        return tuple(grads)
+    if (h is None) == (ckpt is None):
+        raise ValueError("pass exactly one of h and ckpt")
+
+    x, a, b, c, dy = (_unit_inner(t) for t in (x, a, b, c, dy))
+    if h is not None:
+        h = _unit_inner(h if h.dtype == torch.float32 else h.float())
+    else:
+        ckpt = ckpt.contiguous()
+    align = _align_elems([x, a, b, c, dy, h, *grads], D)
+    plan = make_plan(B, L, D, in_dtype, dy.dtype, _lib.QSSM_BACKWARD, align, ckpt_stride if h is None else 0, tune)
+    if ckpt is not None and tuple(ckpt.shape) != (B, plan.n_ckpt, D):
+        raise ValueError(f"ckpt has shape {tuple(ckpt.shape)}, expected {(B, plan.n_ckpt, D)}")
+
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        ws = _workspace(dev, stream, int(plan.workspace_bytes))
+        _lib.check(
+            _lib.load().qssm_scan_backward(
+                ctypes.byref(plan),
+                _ptr(x), _strides(x), _ptr(a), _strides(a), _ptr(b), _strides(b), _ptr(c), _strides(c),
+                _ptr(dy), _strides(dy), _ptr(h), _strides(h), _ptr(ckpt),
+                _ptr(grads[0]), _strides(grads[0]), _ptr(grads[1]), _strides(grads[1]),
+                _ptr(grads[2]), _strides(grads[2]), _ptr(grads[3]), _strides(grads[3]),
+                ws.data_ptr(), ws.numel(), stream,
+            )
+        )
+    return tuple(grads)
+
+
+def block_scan_forward_3d(x: Tensor, a: Tensor, b: Tensor, BLOCK_L: int = 256) -> Tuple[Tensor, Tensor]:
+    """Device forward of h(t) = a(t) h(t-1) + b(t) x(t).
+
+    Same contract as the reference's function of this name (quick_ssm/triton_forwards.py:134-172):
+    3-D GPU inputs, returns fp32 `(out_a, out_x)` with out_x = h and out_a the running product of
+    a.  `BLOCK_L` is accepted for compatibility; the launch geometry no longer depends on it.
+    """
+    for t in (x, a, b):
+        assert t.dim() == 3, "All inputs should be [B, L, D]."
+        assert t.device.type == "cuda", "Inputs must be on a GPU device."
+    B, L, D = x.shape
+    if L == 0:
+        return torch.empty_like(a), torch.empty_like(x)
+    k_in, _ = kernel_dtypes([x.dtype, a.dtype, b.dtype], torch.float32)
+    xs, as_, bs = (t if t.dtype == k_in else t.to(k_in) for t in (x, a, b))
+    h, _, _, _ = scan_forward(xs, as_, bs, None, out_dtype=torch.float32, want_ckpt=False)
+    # out_a is discarded by every caller of the reference; it is kept for the tuple's shape.
+    out_a = torch.cumprod(a.to(torch.float32), dim=1)
+    return out_a, h
+
+
+def block_scan_backward_3d(a: Tensor, b: Tensor, c: Tensor, x: Tensor, h: Tensor, grad_y: Tensor,
+                           BLOCK_L: int = 256) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+    """Device backward given the forward states h; returns fp32 (dx, da, db, dc).
+
+    Same contract and argument order as the reference's function of this name
+    (quick_ssm/triton_backwards.py:168-209), which upcasts every operand to fp32 first.
+    """
+    for t in (a, b, c, x, h, grad_y):
+        assert t.dim() == 3, "All inputs should be [B, L, D]."
+        assert t.device.type == "cuda", "Inputs must be on a GPU device."
+    B, L, D = x.shape
+    if L == 0:
+        return (torch.empty_like(x), torch.empty_like(a), torch.empty_like(b), torch.empty_like(c))
+    f32 = torch.float32
+    a, b, c, x, h, grad_y = (t if t.dtype == f32 else t.to(f32) for t in (a, b, c, x, h, grad_y))
+    return scan_backward(x, a, b, c, grad_y, h=h)

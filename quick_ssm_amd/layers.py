@@ -1,0 +1,99 @@
+"""`SSM` and `RMSNorm`: the layer that feeds the scan.
+
+Same constructor arguments, parameter names (so state dicts interchange) and forward keywords as
+the reference's quick_ssm/layers.py:9-107.  The projections and gate activations stay on torch
+GEMMs / elementwise ops; only the scan inside is the HIP path.  Roles of the projections
+(quick_ssm/test_swiglu_equiv.py:60-70): A_proj -> forget gate a, B_proj -> the scan's input x,
+D_proj -> input gate b, C_proj_a/C_proj_b -> SwiGLU output gate c, out_proj -> output.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .scan_interface import scan
+
+
+class RMSNorm(nn.Module):
+    """x * weight / sqrt(mean(x^2) + eps) over the last axis (quick_ssm/layers.py:9-17)."""
+
+    def __init__(self, hidden_size: int, eps: float = 1e-5, dtype=torch.float32, device=None):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(hidden_size, dtype=dtype, device=device))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        rms = torch.sqrt(x.pow(2).mean(dim=-1, keepdim=True) + self.eps)
+        return x * (self.weight / rms)
+
+
+class SSM(nn.Module):
+    """Gated linear recurrence layer: norm -> five projections -> scan -> out projection (+ residual)."""
+
+    def __init__(
+        self,
+        hidden_size: int,
+        state_size_mult: float = 1.0,
+        eps: float = 1e-5,
+        dtype: torch.dtype = torch.float32,
+        device: Optional[torch.device] = None,
+        compute_dtype: torch.dtype = torch.float16,
+        use_residual: bool = True,
+        use_norm: bool = True,
+    ):
+        super().__init__()
+        self.hidden_size = hidden_size
+        self.state_size_dim = int(hidden_size * state_size_mult)
+        self.compute_dtype = compute_dtype
+        self.use_residual = use_residual
+        self.use_norm = use_norm
+
+        def proj(n_in: int, n_out: int, bias: bool) -> nn.Linear:
+            return nn.Linear(n_in, n_out, bias=bias, device=device, dtype=dtype)
+
+        # Creation order matches the reference so that seeded initialisation matches too.
+        self.A_proj = proj(hidden_size, self.state_size_dim, True)
+        self.B_proj = proj(hidden_size, self.state_size_dim, False)
+        self.C_proj_a = proj(hidden_size, self.state_size_dim, False)
+        self.C_proj_b = proj(hidden_size, self.state_size_dim, False)
+        self.D_proj = proj(hidden_size, self.state_size_dim, False)
+        self.out_proj = proj(self.state_size_dim, hidden_size, True)
+        self.pre_norm = RMSNorm(hidden_size, eps=eps, dtype=dtype, device=device) if use_norm else nn.Identity()
+
+    def gates(self, u: torch.Tensor):
+        """The scan's four operands (x, a, b, c) from the normalised input, in `compute_dtype`."""
+        dt = self.compute_dtype
+        forget = torch.sigmoid(self.A_proj(u)).to(dt)
+        drive = self.B_proj(u).to(dt)
+        out_gate = (F.silu(self.C_proj_a(u)) * self.C_proj_b(u)).to(dt)
+        in_gate = torch.sigmoid(self.D_proj(u)).to(dt)
+        return drive, forget, in_gate, out_gate
+
+    def forward(
+        self,
+        x: torch.Tensor,
+        *,
+        block_l: int = 256,
+        checkpoint: bool = True,
+        tile_b: Optional[int] = None,
+        tile_d: Optional[int] = None,
+        backend: str = "auto",
+        scan_out_dtype: Optional[torch.dtype] = None,
+    ) -> torch.Tensor:
+        skip = x if self.use_residual else 0
+        u = self.pre_norm(x) if self.use_norm else x
+        drive, forget, in_gate, out_gate = self.gates(u)
+        w_dtype = self.out_proj.weight.dtype
+        y = scan(
+            x=drive, a=forget, b=in_gate, c=out_gate,
+            block_l=block_l, checkpoint=checkpoint, tile_b=tile_b, tile_d=tile_d,
+            out_dtype=w_dtype if scan_out_dtype is None else scan_out_dtype,
+            backend=backend,
+        )
+        return self.out_proj(y.to(w_dtype)) + skip
+
+
+__all__ = ["SSM", "RMSNorm"]

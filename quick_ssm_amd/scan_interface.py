@@ -1,0 +1,198 @@
+"""Public scan entry point: `scan(x, a, b, c, *, block_l, checkpoint, tile_b, tile_d, backend, out_dtype)`.
+
+    h(t) = a(t) * h(t-1) + b(t) * x(t)        (all tensors [B, L, D])
+    y(t) = c(t) * h(t)
+
+Same surface as the reference's `quick_ssm/scan_interface.py` (`scan` :169-213, the autograd
+Function :49-158, `_chunk_ranges` :36-46, `_torch_scan` :161-166); the device work behind it is one
+HIP launch per direction on gfx950 instead of Triton kernels inside a Python tile loop.
+
+What the knobs mean here
+  block_l     accepted and recorded.  The kernels pick their own time tiling (tile length and
+              the spacing of the states kept for the backward); results do not depend on it.
+  checkpoint  True: the forward keeps only the fp32 state at every `ckpt_stride`-th step (about
+              1/64 of one tensor) and the backward rebuilds h inside each tile.  False: the
+              forward also keeps the full fp32 h (`ctx.h_saved`, as the reference does) and the
+              backward reads it.
+  tile_b/d    accepted.  They bound the reference's N-sized fp32 scratch, which does not exist
+              here, and rows (b, d) are independent, so by default one launch covers the whole
+              tensor.  `honor_tiles(True)` makes every tile its own launch on a strided view
+              (no copies); results are bitwise the same either way.
+  backend     "auto": the HIP kernels for GPU tensors, the sequential torch recurrence for CPU
+              tensors.  "triton" is kept as the legacy name of the device path, "hip" is its
+              proper name.  "torch": the sequential recurrence on whatever device the tensors
+              are on.  A GPU tensor never takes the sequential path unless "torch" is asked for
+              by name, and the device path raises if libquick_ssm_hip.so is not built.
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Tuple
+
+import torch
+
+from . import hip_scan
+from .naive_baseline import naive_forward_3d
+
+Tensor = torch.Tensor
+
+_HONOR_TILES = False
+
+
+def honor_tiles(flag: bool) -> bool:
+    """Launch once per (tile_b, tile_d) tile instead of once per call.  Returns the old setting."""
+    global _HONOR_TILES
+    old, _HONOR_TILES = _HONOR_TILES, bool(flag)
+    return old
+
+
+def _chunk_ranges(total: int, tile: Optional[int]) -> List[Tuple[int, int]]:
+    """Half-open ranges covering [0, total); no tile, a non-positive one or one >= total gives one range."""
+    if tile is None or tile <= 0 or tile >= total:
+        return [(0, total)]
+    edges = list(range(0, total, tile)) + [total]
+    return list(zip(edges[:-1], edges[1:]))
+
+
+def _launch_tiles(shape, tile_b, tile_d) -> List[Tuple[slice, slice]]:
+    if not _HONOR_TILES:
+        return [(slice(0, shape[0]), slice(0, shape[2]))]
+    return [
+        (slice(b0, b1), slice(d0, d1))
+        for b0, b1 in _chunk_ranges(shape[0], tile_b)
+        for d0, d1 in _chunk_ranges(shape[2], tile_d)
+    ]
+
+
+class _HipScanFunction(torch.autograd.Function):
+    """Autograd node of the device scan: one HIP launch forward, one backward.
+
+    Argument list, saved state and returned gradients follow the reference's
+    `_TritonScanFunction` (quick_ssm/scan_interface.py:49-158): forward takes
+    (x, a, b, c, block_l, checkpoint, tile_b, tile_d, out_dtype); backward returns
+    (dx, da, db, dc, None x 5) with every gradient in its operand's dtype.
+    """
+
+    @staticmethod
+    def forward(ctx, x: Tensor, a: Tensor, b: Tensor, c: Tensor, block_l: int, checkpoint: bool,
+                tile_b: Optional[int], tile_d: Optional[int], out_dtype: torch.dtype) -> Tensor:
+        if x.shape != a.shape or x.shape != b.shape or x.shape != c.shape:
+            raise ValueError("x, a, b, c must share the same shape [B, L, D].")
+        if x.dim() != 3:
+            raise ValueError("x, a, b, c must be 3-D tensors [B, L, D].")
+        if x.device.type != "cuda":
+            raise RuntimeError("HIP scan backend requires GPU tensors.")
+
+        ctx.block_l = int(block_l)
+        ctx.checkpoint = bool(checkpoint)
+        ctx.tile_b = tile_b
+        ctx.tile_d = tile_d
+        ctx.out_dtype = out_dtype
+        ctx.save_for_backward(x, a, b, c)
+
+        k_in, k_out = hip_scan.kernel_dtypes([x.dtype, a.dtype, b.dtype, c.dtype], out_dtype)
+        xs, as_, bs, cs = (t if t.dtype == k_in else t.to(k_in) for t in (x, a, b, c))
+        ctx.k_in, ctx.k_out = k_in, k_out
+
+        tiles = _launch_tiles(x.shape, tile_b, tile_d)
+        ctx.tiles = tiles
+        ctx.tile_states = []
+        whole = len(tiles) == 1
+        y = None if whole else torch.empty(x.shape, dtype=k_out, device=x.device)
+        h_saved = None
+        if not checkpoint and not whole:
+            h_saved = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+        for bs_, ds_ in tiles:
+            yt, ht, ckpt, stride = hip_scan.scan_forward(
+                xs[bs_, :, ds_], as_[bs_, :, ds_], bs[bs_, :, ds_], cs[bs_, :, ds_],
+                out_dtype=k_out, want_h=not checkpoint, want_ckpt=bool(checkpoint),
+            )
+            ctx.tile_states.append((ckpt, stride))
+            if whole:
+                y, h_saved = yt, ht
+            else:
+                y[bs_, :, ds_] = yt
+                if h_saved is not None:
+                    h_saved[bs_, :, ds_] = ht
+        ctx.h_saved = h_saved
+        return y if y.dtype == out_dtype else y.to(out_dtype)
+
+    @staticmethod
+    def backward(ctx, grad_output: Tensor):
+        x, a, b, c = ctx.saved_tensors
+        k_in, k_out = ctx.k_in, ctx.k_out
+        xs, as_, bs, cs = (t if t.dtype == k_in else t.to(k_in) for t in (x, a, b, c))
+        dy = grad_output if grad_output.dtype == k_out else grad_output.to(k_out)
+        need = tuple(ctx.needs_input_grad[:4])
+
+        whole = len(ctx.tiles) == 1
+        grads = [None, None, None, None]
+        if not whole:
+            grads = [torch.empty(x.shape, dtype=k_in, device=x.device) if n else None for n in need]
+        for (bs_, ds_), (ckpt, stride) in zip(ctx.tiles, ctx.tile_states):
+            h_tile = None if ctx.h_saved is None else ctx.h_saved[bs_, :, ds_]
+            out = hip_scan.scan_backward(
+                xs[bs_, :, ds_], as_[bs_, :, ds_], bs[bs_, :, ds_], cs[bs_, :, ds_], dy[bs_, :, ds_],
+                h=h_tile, ckpt=None if h_tile is not None else ckpt, ckpt_stride=stride, need=need,
+            )
+            if whole:
+                grads = list(out)
+            else:
+                for gfull, gt in zip(grads, out):
+                    if gfull is not None:
+                        gfull[bs_, :, ds_] = gt
+
+        def _as(g: Optional[Tensor], like: Tensor) -> Optional[Tensor]:
+            if g is None:
+                return None
+            return g if g.dtype == like.dtype else g.to(like.dtype)
+
+        return (_as(grads[0], x), _as(grads[1], a), _as(grads[2], b), _as(grads[3], c),
+                None, None, None, None, None)
+
+
+# The reference's name for the autograd node; kept so that code reaching for it still works.
+_TritonScanFunction = _HipScanFunction
+
+
+def _torch_scan(x: Tensor, a: Tensor, b: Tensor, c: Tensor, out_dtype: torch.dtype) -> Tensor:
+    """Sequential recurrence in plain torch (the reference's CPU path, scan_interface.py:161-166)."""
+    h = naive_forward_3d(x, a, b)
+    return (c * h).to(out_dtype)
+
+
+def scan(
+    x: Tensor,
+    a: Tensor,
+    b: Tensor,
+    c: Tensor,
+    *,
+    block_l: int = 256,
+    checkpoint: bool = True,
+    tile_b: Optional[int] = None,
+    tile_d: Optional[int] = None,
+    backend: str = "auto",
+    out_dtype: Optional[torch.dtype] = None,
+) -> Tensor:
+    """Gated linear scan y = c * h, h(t) = a(t) h(t-1) + b(t) x(t), differentiable in x, a, b, c.
+
+    Args:
+        x, a, b, c: tensors of shape [B, L, D].
+        block_l, checkpoint, tile_b, tile_d: see the module docstring.
+        backend: "auto" (default), "hip" / "triton" (device kernels), or "torch".
+        out_dtype: dtype of the returned tensor; defaults to x.dtype.
+
+    Returns:
+        y of shape [B, L, D] and dtype `out_dtype`.
+    """
+    out_dtype = out_dtype or x.dtype
+    chosen = backend
+    if backend == "auto":
+        chosen = "hip" if x.device.type == "cuda" else "torch"
+    if chosen in ("hip", "triton"):
+        return _HipScanFunction.apply(x, a, b, c, block_l, checkpoint, tile_b, tile_d, out_dtype)
+    if chosen == "torch":
+        return _torch_scan(x, a, b, c, out_dtype)
+    raise ValueError(f"Unsupported backend '{backend}'. Use 'auto', 'hip', 'triton', or 'torch'.")
+
+
+__all__ = ["scan", "honor_tiles"]

@@ -1,0 +1,165 @@
+"""Pins the CPU oracle (oracle/) before anything is compared with it.
+
+Checks chosen so that a dropped term, a wrong sign or index, or a transposed operand fails one:
+exact rational vectors from the scan's definition as an explicit sum (tests/golden), closed forms,
+finite differences, structural invariants, and agreement between the independently written C and
+torch flavours.  None of these retypes the oracle's recurrence.
+"""
+import json
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle.reference_cpu_path import reference_forward_states, reference_scan, reference_scan_with_grads
+from helpers import make_inputs, oracle_all
+
+GOLDEN = json.loads((Path(__file__).parent / "golden" / "exact_scan_vectors.json").read_text())
+
+
+@pytest.mark.parametrize("case", GOLDEN["cases"], ids=lambda c: c["name"])
+def test_oracle_matches_exact_rational_vectors(case):
+    ops = [np.array(case[k], dtype=np.float32) for k in ("x", "a", "b", "c", "dy")]
+    for k, arr in zip(("x", "a", "b", "c", "dy"), ops):  # inputs are exactly representable
+        assert np.array_equal(arr.astype(np.float64), np.array(case[k]))
+    x, a, b, c, dy = ops
+    h, y = oracle.forward_f64(x, a, b, c)
+    grads = dict(zip(("dx", "da", "db", "dc"), oracle.backward_f64(x, a, b, c, dy)))
+    np.testing.assert_allclose(h, np.array(case["h"]), rtol=1e-14, atol=1e-14)
+    np.testing.assert_allclose(y, np.array(case["y"]), rtol=1e-14, atol=1e-14)
+    for k, g in grads.items():
+        np.testing.assert_allclose(g, np.array(case[k]), rtol=1e-13, atol=1e-13, err_msg=k)
+
+
+@pytest.mark.parametrize("case", GOLDEN["cases"], ids=lambda c: c["name"])
+def test_torch_restatement_matches_exact_rational_vectors(case):
+    x, a, b, c, dy = (torch.tensor(case[k], dtype=torch.float64) for k in ("x", "a", "b", "c", "dy"))
+    y, dx, da, db, dc = reference_scan_with_grads(x, a, b, c, dy)
+    for k, got in (("y", y), ("dx", dx), ("da", da), ("db", db), ("dc", dc)):
+        np.testing.assert_allclose(got.numpy(), np.array(case[k]), rtol=1e-13, atol=1e-13, err_msg=k)
+
+
+def test_closed_form_geometric_decay():
+    # x = delta(t=0), b = 1, a = g  =>  h(t) = g^t  (the reference's precision test, forward_only.py:592-600,
+    # at a length where g^L stays a normal number)
+    L, g = 4096, 0.999
+    x = np.zeros((1, L, 2), np.float32)
+    x[:, 0] = 1.0
+    a = np.full_like(x, g)
+    b = np.ones_like(x)
+    h, _ = oracle.forward_f64(x, a, b)
+    expect = np.float64(np.float32(g)) ** np.arange(L)
+    np.testing.assert_allclose(h[0, :, 0], expect, rtol=1e-12)
+
+
+def test_closed_forms_cumsum_and_memoryless_and_geometric_sum():
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((2, 300, 3)).astype(np.float32)
+    b = rng.standard_normal((2, 300, 3)).astype(np.float32)
+    ones, zeros = np.ones_like(x), np.zeros_like(x)
+    h, _ = oracle.forward_f64(x, ones, b)                      # a = 1: running sum of b*x
+    np.testing.assert_allclose(h, np.cumsum(b.astype(np.float64) * x, axis=1), rtol=1e-12, atol=1e-12)
+    h, _ = oracle.forward_f64(x, zeros, b)                     # a = 0: no memory
+    np.testing.assert_allclose(h, b.astype(np.float64) * x, rtol=0, atol=0)
+    g = np.float32(0.75)
+    h, _ = oracle.forward_f64(ones, np.full_like(x, g), ones)  # a = g, b*x = 1: (1 - g^(t+1)) / (1 - g)
+    t = np.arange(300)
+    np.testing.assert_allclose(h[1, :, 2], (1 - np.float64(g) ** (t + 1)) / (1 - np.float64(g)), rtol=1e-13)
+
+
+def test_gradients_match_finite_differences():
+    x, a, b, c, dy = (t.double().numpy() for t in make_inputs((1, 7, 2), seed=5))
+    f32 = [t.astype(np.float32) for t in (x, a, b, c, dy)]
+    grads = oracle.backward_f64(*f32)
+
+    def loss(ops):
+        _, y = oracle.forward_f64(ops[0], ops[1], ops[2], ops[3])
+        return float((y * f32[4].astype(np.float64)).sum())
+
+    # the loss is affine in each single input, so a wide central difference is exact up to rounding
+    step = np.float32(0.25)
+    for which, g in enumerate(grads):
+        for idx in np.ndindex(f32[which].shape):
+            hi = [t.copy() for t in f32[:4]]
+            lo = [t.copy() for t in f32[:4]]
+            hi[which][idx] += step
+            lo[which][idx] -= step
+            fd = (loss(hi) - loss(lo)) / (float(hi[which][idx]) - float(lo[which][idx]))  # the step as stored
+            assert abs(fd - g[idx]) <= 1e-9 * max(1.0, abs(fd)), (which, idx, fd, g[idx])
+
+
+def test_gradient_invariants():
+    x, a, b, c, dy = make_inputs((2, 65, 4), seed=9)
+    r = oracle_all(x, a, b, c, dy)
+    h, _ = oracle.forward_f64(x, a, b, c)
+    assert np.all(r["da"][:, 0, :] == 0.0)                                    # h(-1) = 0
+    np.testing.assert_allclose(r["dc"], dy.double().numpy() * h, rtol=1e-14)  # dc = dy * h
+    np.testing.assert_allclose(r["dx"] * x.double().numpy(), r["db"] * b.double().numpy(), rtol=1e-12, atol=1e-15)
+    # linearity of every gradient in dy
+    r2 = oracle_all(x, a, b, c, (2 * dy))
+    for k in ("dx", "da", "db", "dc"):
+        np.testing.assert_allclose(r2[k], 2 * r[k], rtol=1e-14)
+
+
+def test_time_concatenation_property():
+    # scanning [0, L) equals scanning [0, k) and then [k, L) seeded with h(k-1); the seed enters as an
+    # extra drive term a(k) * h(k-1) folded into step k
+    x, a, b, c, _ = make_inputs((1, 40, 3), seed=11)
+    h_full, _ = oracle.forward_f64(x, a, b, c)
+    k = 17
+    h_head, _ = oracle.forward_f64(x[:, :k], a[:, :k], b[:, :k], c[:, :k])
+    x2, b2 = x[:, k:].double().numpy().copy(), b[:, k:].double().numpy().copy()
+    # fold the seed into the first step: b*x + a*h_prev (kept in float64 by passing b = 1, x = drive)
+    drive = b2 * x2
+    drive[:, 0] += a[:, k].double().numpy() * h_head[:, -1]
+    state = np.zeros_like(drive[:, 0])
+    tail = []
+    for t in range(drive.shape[1]):
+        state = (a[:, k + t].double().numpy() if t > 0 else 0.0) * state + drive[:, t]
+        tail.append(state)
+    np.testing.assert_allclose(np.stack(tail, axis=1), h_full[:, k:], rtol=1e-13)
+
+
+def test_c_and_torch_flavours_agree_bitwise_in_fp32():
+    x, a, b, c, dy = make_inputs((2, 130, 5), seed=3)
+    h_c = oracle.forward_f32_seq(x, a, b)
+    h_t = reference_forward_states(x, a, b)
+    assert np.array_equal(h_c, h_t.numpy())
+    y, dx, da, db, dc = reference_scan_with_grads(x, a, b, c, dy)
+    got = oracle.backward_f32_seq(x, a, b, c, dy, h_c)
+    # autograd accumulates the same products; sums of two terms may associate differently only in dH,
+    # where both sides add (dy*c) + carried term in that order
+    for name, g_c, g_t in zip(("dx", "da", "db", "dc"), got, (dx, da, db, dc)):
+        np.testing.assert_allclose(g_c, g_t.numpy(), rtol=2e-6, atol=1e-7, err_msg=name)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_torch_restatement_rounding_points(dtype):
+    # 16-bit inputs: fp32 accumulation, h rounded to the input dtype, then c*h in the input dtype
+    x, a, b, c, _ = make_inputs((1, 33, 4), dtype=dtype, seed=4)
+    h64, _ = oracle.forward_f64(x, a, b, c)
+    h = reference_forward_states(x, a, b)
+    assert h.dtype == dtype
+    expect_h = torch.from_numpy(oracle.forward_f32_seq(x, a, b)).to(dtype)
+    assert torch.equal(h, expect_h)
+    y = reference_scan(x, a, b, c)
+    assert torch.equal(y, c * expect_h)
+    assert oracle.error_report(y, h64 * c.double().numpy())["scaled"] < 1e-2
+
+
+def test_product_cpu_path_equals_reference_cpu_path():
+    # quick_ssm_amd's own backend="torch" path advances all batch rows at once; element for element it
+    # must do what the reference's loop does
+    from quick_ssm_amd.scan_interface import scan
+
+    for dtype in (torch.float32, torch.float16, torch.bfloat16):
+        x, a, b, c, dy = make_inputs((3, 70, 6), dtype=dtype, seed=8)
+        leaves = [t.clone().requires_grad_(True) for t in (x, a, b, c)]
+        y = scan(*leaves, backend="torch")
+        y.backward(dy)
+        y_ref, *g_ref = reference_scan_with_grads(x, a, b, c, dy)
+        assert torch.equal(y, y_ref)
+        for t, g in zip(leaves, g_ref):
+            assert torch.allclose(t.grad.float(), g.float(), rtol=1e-5, atol=1e-6)

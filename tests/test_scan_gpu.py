@@ -1,0 +1,325 @@
+"""Parity of the HIP scan (through the C ABI) with the CPU oracle, on a real MI355X.
+
+Bar: per tensor, max|got - oracle| / max|oracle| <= 1e-5 for fp32 storage and <= 1e-2 for fp16 / bf16
+storage, the oracle being float64 arithmetic on the same stored inputs.  fp32 cases are also held
+to the reference tests' own allclose(rtol=1e-3, atol=1e-5) against the fp32 sequential recurrence.
+"""
+import json
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import TOL, assert_close, make_inputs, oracle_all, run_scan_with_grads
+from quick_ssm_amd import hip_scan
+from quick_ssm_amd.scan_interface import honor_tiles, scan
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = json.loads((Path(__file__).parent / "golden" / "exact_scan_vectors.json").read_text())
+
+
+def _check_all(got, ref, tol):
+    report = {}
+    for k in ("y", "dx", "da", "db", "dc"):
+        assert_close(k, got[k], ref[k], tol, report)
+    return report
+
+
+# ---- the reference's own test cases ----------------------------------------------------------------
+
+@pytest.mark.parametrize("shape,block_l,seed", [((2, 512, 8), 128, 42), ((1, 4, 1), 8, 3), ((1, 1024, 1), 1024, 4)])
+def test_forward_cases_of_reference_test_forwards(gpu, shape, block_l, seed):
+    # quick_ssm/test_forwards.py:108-114: fp32 h against the sequential recurrence, rtol 1e-3 atol 1e-5
+    x, a, b, _, _ = make_inputs(shape, seed=seed)
+    print(f"case fwd shape={shape} block_l={block_l} seed={seed}", flush=True)
+    out_a, h = hip_scan.block_scan_forward_3d(x.to(gpu), a.to(gpu), b.to(gpu), BLOCK_L=block_l)
+    assert h.dtype == torch.float32 and out_a.shape == h.shape
+    h_seq = torch.from_numpy(oracle.forward_f32_seq(x, a, b))
+    assert torch.allclose(h.cpu(), h_seq, rtol=1e-3, atol=1e-5)
+    h64, _ = oracle.forward_f64(x, a, b)
+    assert_close("h", h, h64, 1e-5)
+    assert_close("out_a", out_a, np.cumprod(a.double().numpy(), axis=1), 1e-5)
+
+
+@pytest.mark.parametrize("shape", [(2, 2048, 8), (1, 1024, 1)])
+def test_backward_cases_of_reference_test_backwards(gpu, shape):
+    # quick_ssm/test_backwards.py:120-125: b, c ~ N(0,1), h from the sequential recurrence fed in, fp32
+    x, a, b, c, dy = make_inputs(shape, seed=0, unit_bc=True)
+    print(f"case bwd shape={shape}", flush=True)
+    h_seq = torch.from_numpy(oracle.forward_f32_seq(x, a, b))
+    got = hip_scan.block_scan_backward_3d(*(t.to(gpu) for t in (a, b, c, x, h_seq, dy)))
+    ref = oracle.backward_f64(x, a, b, c, dy)
+    seq = oracle.backward_f32_seq(x, a, b, c, dy, h_seq)
+    for name, g, r, s in zip(("dx", "da", "db", "dc"), got, ref, seq):
+        assert g.dtype == torch.float32
+        assert_close(name, g, r, 1e-5)
+        assert torch.allclose(g.cpu(), torch.from_numpy(s), rtol=1e-3, atol=1e-5 * max(1.0, float(np.abs(r).max())))
+
+
+def test_scan_interface_case_of_reference(gpu):
+    # quick_ssm/test_scan_interface.py:8-31: B2 L32 D4, block_l 16, fp16 on the device, grads within atol 1e-4 rtol 1e-3
+    # of the sequential path (here: of the float64 oracle, at the fp16 bar)
+    x, a, b, c, dy = make_inputs((2, 32, 4), dtype=torch.float16, seed=0)
+    got = run_scan_with_grads(scan, x, a, b, c, dy, gpu, block_l=16, checkpoint=True)
+    _check_all(got, oracle_all(x, a, b, c, dy), TOL[torch.float16])
+
+
+# ---- exact vectors and closed forms -----------------------------------------------------------------
+
+@pytest.mark.parametrize("case", GOLDEN["cases"], ids=lambda c: c["name"])
+def test_exact_rational_vectors(gpu, case):
+    x, a, b, c, dy = (torch.tensor(case[k], dtype=torch.float32) for k in ("x", "a", "b", "c", "dy"))
+    got = run_scan_with_grads(scan, x, a, b, c, dy, gpu)
+    for k in ("y", "dx", "da", "db", "dc"):
+        np.testing.assert_allclose(got[k].double().numpy(), np.array(case[k]), rtol=2e-6, atol=2e-6, err_msg=k)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_closed_form_geometric_decay(gpu, dtype):
+    # x = delta(t=0), b = 1, a = g: h(t) = g^t (the idea of quick_ssm/forward_only.py:548-629)
+    L, g = 4096, 0.999
+    x = torch.zeros(1, L, 2, dtype=dtype)
+    x[:, 0] = 1
+    a = torch.full_like(x, g)
+    b = torch.ones_like(x)
+    _, h = hip_scan.block_scan_forward_3d(x.to(gpu), a.to(gpu), b.to(gpu))
+    g_stored = float(a[0, 0, 0].double())
+    expect = g_stored ** np.arange(L)
+    rel = np.abs(h[0, :, 0].double().cpu().numpy() - expect) / expect
+    assert rel.max() < (1e-5 if dtype == torch.float32 else 1e-2) * 30  # error grows with t; ~L * eps / 2
+    assert rel[-1] < 3e-4
+
+
+# ---- shapes, dtypes, edges ---------------------------------------------------------------------------
+
+SHAPES = [
+    (4, 2048, 16),    # config 0
+    (2, 300, 5),      # ragged L, odd D (1 column per lane)
+    (1, 1, 1),
+    (3, 7, 2),
+    (2, 1000, 6),     # D multiple of 2 only
+    (2, 777, 64),     # several tiles per chain, ragged last tile
+    (1, 4096, 128),
+    (2, 1500, 260),   # two strips, the second partial
+    (5, 64, 1024),    # config 4's per-layer shape (smaller batch)
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=["f32", "f16", "bf16"])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_scan_matches_oracle(gpu, shape, dtype):
+    x, a, b, c, dy = make_inputs(shape, dtype=dtype, seed=sum(shape))
+    print(f"case scan shape={shape} dtype={dtype}", flush=True)
+    got = run_scan_with_grads(scan, x, a, b, c, dy, gpu)
+    assert got["y"].dtype == dtype and got["dx"].dtype == dtype
+    _check_all(got, oracle_all(x, a, b, c, dy), TOL[dtype])
+    assert torch.all(got["da"][:, 0, :] == 0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+def test_fp32_output_from_16bit_operands(gpu, dtype):
+    # what SSM does with fp32 parameters: 16-bit operands, y and dy in fp32 (quick_ssm/layers.py:85-91)
+    x, a, b, c, dy = make_inputs((2, 700, 96), dtype=dtype, seed=21, out_dtype=torch.float32)
+    got = run_scan_with_grads(scan, x, a, b, c, dy, gpu, out_dtype=torch.float32)
+    assert got["y"].dtype == torch.float32 and got["da"].dtype == dtype
+    ref = oracle_all(x, a, b, c, dy)
+    assert_close("y", got["y"], ref["y"], 1e-5)  # fp32 storage of y: only fp32 arithmetic error remains
+    for k in ("dx", "da", "db", "dc"):
+        assert_close(k, got[k], ref[k], TOL[dtype])
+
+
+def test_mixed_operand_dtypes_and_unbuilt_output_dtype(gpu):
+    x, a, b, c, dy = make_inputs((2, 130, 8), seed=2)
+    a16, c16 = a.to(torch.float16), c.to(torch.bfloat16)
+    got = run_scan_with_grads(scan, x, a16, b, c16, dy.to(torch.float16), gpu, out_dtype=torch.float16)
+    assert got["y"].dtype == torch.float16
+    assert got["da"].dtype == torch.float16 and got["dc"].dtype == torch.bfloat16 and got["dx"].dtype == torch.float32
+    ref = oracle_all(x, a16, b, c16, dy.to(torch.float16))
+    for k in ("y", "dx", "da", "db", "dc"):
+        assert_close(k, got[k], ref[k], 1e-2)
+
+
+def test_empty_sequence_and_empty_batch(gpu):
+    for shape in [(2, 0, 4), (0, 5, 4), (2, 5, 0)]:
+        x = torch.zeros(shape, device=gpu, requires_grad=True)
+        y = scan(x, x.detach(), x.detach(), x.detach())
+        assert y.shape == torch.Size(shape)
+        y.sum().backward()
+        assert x.grad.shape == torch.Size(shape)
+    o_a, o_x = hip_scan.block_scan_forward_3d(*(torch.zeros(1, 0, 3, device=gpu) for _ in range(3)))
+    assert o_a.shape == (1, 0, 3) and o_x.shape == (1, 0, 3)
+
+
+def test_non_contiguous_operands(gpu):
+    shape = (3, 200, 24)
+    x, a, b, c, dy = make_inputs(shape, seed=5)
+    ref = oracle_all(x, a, b, c, dy)
+    dev = [t.to(gpu) for t in (x, a, b, c)]
+    big = torch.zeros(3, 400, 48, device=gpu)
+    big[:, ::2, 8:32] = dev[0]
+    views = [
+        big[:, ::2, 8:32],                                      # strided in time, offset in D
+        dev[1].transpose(0, 1).contiguous().transpose(0, 1),    # batch and time swapped in memory
+        dev[2].permute(0, 2, 1).contiguous().permute(0, 2, 1),  # D not the fast axis: copied by the host
+        dev[3][:, :, :],
+    ]
+    leaves = [v.detach().requires_grad_(True) for v in views]
+    y = scan(*leaves)
+    y.backward(dy.to(gpu).expand_as(y))
+    got = {"y": y.detach().cpu()}
+    for k, t in zip(("dx", "da", "db", "dc"), leaves):
+        got[k] = t.grad.cpu()
+    _check_all(got, ref, 1e-5)
+
+
+# ---- knobs must not change results ---------------------------------------------------------------------
+
+def test_checkpoint_false_keeps_fp32_states_and_matches(gpu):
+    x, a, b, c, dy = make_inputs((2, 900, 40), dtype=torch.float16, seed=6)
+    on = run_scan_with_grads(scan, x, a, b, c, dy, gpu, checkpoint=True)
+    off = run_scan_with_grads(scan, x, a, b, c, dy, gpu, checkpoint=False)
+    assert torch.equal(on["y"], off["y"])
+    ref = oracle_all(x, a, b, c, dy)
+    _check_all(off, ref, TOL[torch.float16])
+    # the saved states themselves
+    leaves = [t.to(gpu).requires_grad_(True) for t in (x, a, b, c)]
+    y = scan(*leaves, checkpoint=False)
+    h_saved = y.grad_fn.h_saved
+    assert h_saved is not None and h_saved.dtype == torch.float32
+    h64, _ = oracle.forward_f64(x, a, b, c)
+    assert_close("h_saved", h_saved, h64, 1e-5)
+    y2 = scan(*leaves, checkpoint=True)
+    assert y2.grad_fn.h_saved is None
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_block_l_and_tiles_do_not_change_results(gpu, dtype):
+    x, a, b, c, dy = make_inputs((4, 600, 48), dtype=dtype, seed=7)
+    base = run_scan_with_grads(scan, x, a, b, c, dy, gpu)
+    for block_l in (1, 7, 16, 256, 4096):
+        other = run_scan_with_grads(scan, x, a, b, c, dy, gpu, block_l=block_l, tile_b=1, tile_d=16)
+        for k in base:
+            assert torch.equal(base[k], other[k]), (block_l, k)
+    old = honor_tiles(True)
+    try:
+        for tb, td in ((1, 16), (3, 20), (None, 8), (2, None)):
+            tiled = run_scan_with_grads(scan, x, a, b, c, dy, gpu, tile_b=tb, tile_d=td)
+            for k in base:
+                assert torch.equal(base[k], tiled[k]), (tb, td, k)
+    finally:
+        honor_tiles(old)
+
+
+def test_launch_geometry_does_not_change_results_beyond_rounding(gpu):
+    # every lanes-per-row / steps-per-lane geometry must agree with the oracle
+    x, a, b, c, dy = make_inputs((2, 1100, 72), seed=8)
+    ref = oracle_all(x, a, b, c, dy)
+    dev = [t.to(gpu) for t in (x, a, b, c)]
+    for g_log2 in (0, 2, 4, 5, 6, 8):
+        for steps in (4, 8):
+            tune = (g_log2 + 1) | (steps << 8)
+            y, _, ckpt, stride = hip_scan.scan_forward(*dev, out_dtype=torch.float32, tune=tune, bwd_tune=tune)
+            grads = hip_scan.scan_backward(*dev, dy.to(gpu), ckpt=ckpt, ckpt_stride=stride, tune=tune)
+            got = dict(zip(("y", "dx", "da", "db", "dc"), (y,) + grads))
+            print(f"geometry g_log2={g_log2} steps={steps} ckpt_stride={stride}", flush=True)
+            _check_all(got, ref, 1e-5)
+
+
+def test_partial_gradients(gpu):
+    x, a, b, c, dy = make_inputs((2, 400, 16), seed=9)
+    ref = oracle_all(x, a, b, c, dy)
+    xs = x.to(gpu).requires_grad_(True)
+    cs = c.to(gpu).requires_grad_(True)
+    y = scan(xs, a.to(gpu), b.to(gpu), cs)
+    y.backward(dy.to(gpu))
+    assert_close("dx", xs.grad, ref["dx"], 1e-5)
+    assert_close("dc", cs.grad, ref["dc"], 1e-5)
+
+
+def test_argument_errors(gpu):
+    x = torch.zeros(2, 8, 4, device=gpu)
+    with pytest.raises(ValueError):
+        scan(x, x[:, :4], x, x)
+    with pytest.raises(ValueError):
+        scan(x, x, x, x, backend="cuda")
+    with pytest.raises(RuntimeError):
+        scan(x.cpu(), x.cpu(), x.cpu(), x.cpu(), backend="triton")
+
+
+# ---- the headline shapes ---------------------------------------------------------------------------------
+
+def _rows_check(got, ops, dy, rows, tol):
+    """Compare whole batch rows (all of L and D) of every output with the oracle."""
+    x, a, b, c = ops
+    for r in rows:
+        sl = slice(r, r + 1)
+        ref = oracle_all(x[sl], a[sl], b[sl], c[sl], dy[sl])
+        for k in ("y", "dx", "da", "db", "dc"):
+            assert_close(f"{k}[row {r}]", got[k][sl], ref[k], tol)
+
+
+def test_config1_bf16_full_shape(gpu):
+    # B=8 L=4096 D=2048 bf16: batch rows 0 and 7 against the oracle over every tile of their chains, the
+    # rest through properties that hold at any size
+    shape = (8, 4096, 2048)
+    x, a, b, c, dy = make_inputs(shape, dtype=torch.bfloat16, seed=0)
+    print("case config1 full shape", flush=True)
+    got = run_scan_with_grads(scan, x, a, b, c, dy, gpu, block_l=256, checkpoint=True)
+    _rows_check(got, (x, a, b, c), dy, (0, 7), TOL[torch.bfloat16])
+    assert torch.all(got["da"][:, 0, :] == 0)
+    for k in got:
+        assert torch.isfinite(got[k].float()).all(), k
+    # dx * x and db * b are the same number b*x*dH up to one rounding each
+    lhs = got["dx"].float() * x.float()
+    rhs = got["db"].float() * b.float()
+    assert torch.allclose(lhs, rhs, rtol=2e-2, atol=1e-6)
+    # linearity in dy: doubling dy doubles every gradient exactly (power of two)
+    twice = run_scan_with_grads(scan, x, a, b, c, dy * 2, gpu)
+    for k in ("dx", "da", "db", "dc"):
+        assert torch.equal(twice[k].float(), got[k].float() * 2), k
+    assert hip_scan.workspace_status() == 0
+
+
+def test_config2_fp16_long_sequence_near_unit_decay(gpu):
+    # B=1 L=65536 D=4096 fp16, a in [0.99, 1], block_l=1024, tile_d=1024: first and last 64 columns over all of L
+    shape = (1, 65536, 4096)
+    x, a, b, c, dy = make_inputs(shape, dtype=torch.float16, seed=1, a_lo=0.99, a_span=0.01)
+    print("case config2 full shape", flush=True)
+    got = run_scan_with_grads(scan, x, a, b, c, dy, gpu, block_l=1024, checkpoint=True, tile_d=1024)
+    for cols in (slice(0, 64), slice(4032, 4096)):
+        ref = oracle_all(x[..., cols], a[..., cols], b[..., cols], c[..., cols], dy[..., cols])
+        for k in ("y", "dx", "da", "db", "dc"):
+            assert_close(f"{k}[cols {cols.start}:{cols.stop}]", got[k][..., cols], ref[k], TOL[torch.float16])
+    for k in got:
+        assert torch.isfinite(got[k].float()).all(), k
+    assert hip_scan.workspace_status() == 0
+
+
+def test_config3_ssm_layer_matches_sequential_path(gpu):
+    # SSM(hidden, state = 4*hidden), fp32 parameters, fp16 scan operands, fp32 scan output; the device layer
+    # against the same layer on the sequential torch path (smaller than config 3 so the CPU side takes seconds)
+    from quick_ssm_amd.layers import SSM
+
+    torch.manual_seed(0)
+    layer = SSM(hidden_size=64, state_size_mult=4.0, compute_dtype=torch.float16, dtype=torch.float32)
+    xin = torch.randn(2, 192, 64)
+    gout = torch.randn(2, 192, 64)
+
+    def run(mod, inp, backend):
+        mod.zero_grad(set_to_none=True)
+        inp = inp.clone().requires_grad_(True)
+        out = mod(inp, backend=backend)
+        out.backward(gout.to(inp.device))
+        grads = {n: p.grad.detach().cpu().clone() for n, p in mod.named_parameters()}
+        return out.detach().cpu(), inp.grad.detach().cpu(), grads
+
+    y_ref, dx_ref, g_ref = run(layer, xin, "torch")
+    layer_gpu = layer.to(gpu)
+    y_gpu, dx_gpu, g_gpu = run(layer_gpu, xin.to(gpu), "auto")
+    assert_close("layer out", y_gpu, y_ref.double().numpy(), 1e-2)
+    assert_close("layer dx", dx_gpu, dx_ref.double().numpy(), 1e-2)
+    for n in g_ref:
+        assert_close(f"grad {n}", g_gpu[n], g_ref[n].double().numpy(), 2e-2)
