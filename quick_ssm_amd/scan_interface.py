@@ -17,7 +17,8 @@ What the knobs mean here
   tile_b/d    accepted.  They bound the reference's N-sized fp32 scratch, which does not exist
               here, and rows (b, d) are independent, so by default one launch covers the whole
               tensor.  `honor_tiles(True)` makes every tile its own launch on a strided view
-              (no copies); results are bitwise the same either way.
+              (no copies); batch tiles give bitwise the same results, feature tiles agree to
+              fp32 rounding (a narrower tile changes how lanes split the time axis).
   backend     "auto": the HIP kernels for GPU tensors, the sequential torch recurrence for CPU
               tensors.  "triton" is kept as the legacy name of the device path, "hip" is its
               proper name.  "torch": the sequential recurrence on whatever device the tensors

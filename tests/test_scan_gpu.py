@@ -203,12 +203,17 @@ def test_block_l_and_tiles_do_not_change_results(gpu, dtype):
         other = run_scan_with_grads(scan, x, a, b, c, dy, gpu, block_l=block_l, tile_b=1, tile_d=16)
         for k in base:
             assert torch.equal(base[k], other[k]), (block_l, k)
+    # One launch per tile: batch tiles keep the launch geometry, so results stay bitwise equal; feature tiles
+    # narrower than a strip change how lanes split the time axis, so results agree to rounding.
+    ref = oracle_all(x, a, b, c, dy)
     old = honor_tiles(True)
     try:
-        for tb, td in ((1, 16), (3, 20), (None, 8), (2, None)):
+        for tb, td in ((1, None), (3, None), (1, 16), (3, 20), (None, 8)):
             tiled = run_scan_with_grads(scan, x, a, b, c, dy, gpu, tile_b=tb, tile_d=td)
-            for k in base:
-                assert torch.equal(base[k], tiled[k]), (tb, td, k)
+            if td is None:
+                for k in base:
+                    assert torch.equal(base[k], tiled[k]), (tb, td, k)
+            _check_all(tiled, ref, TOL[dtype])
     finally:
         honor_tiles(old)
 
