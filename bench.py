@@ -1,0 +1,242 @@
+#!/usr/bin/env python3
+"""Benchmark of the gated linear scan hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c0|c2|c3scan|c4scan]
+
+A step is one forward + backward of `scan()` (the public API, through autograd) over one batch
+of synthetic operands already resident in HBM.  The default workload is the configuration the
+headline metric is quoted on: bf16, B=8, L=4096, D=2048, block_l=256, checkpoint=True.
+
+One JSON line is printed.  `value` is algorithmic HBM bytes per step (forward: read x, a, b, c,
+write y; backward: read x, a, b, c, dy, write dx, da, db, dc; state rebuild and carries count as
+zero) divided by the measured time per step.  `roofline` prices the dominant kernel (the
+backward: 9 of the 14 tensor passes) from HIP-event timing of back-to-back launches on the
+launch stream.  `cpu_baseline` times the torch restatement of the reference's CPU path on a
+bounded slice of the same workload on this box's host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak, 8 TB/s
+
+WORKLOADS = {
+    # name: (B, L, D, operand dtype, y/dy dtype, a_lo, a_span, block_l, description)
+    "c0": (4, 2048, 16, "float32", "float32", 0.9, 0.1, 256, "fp32 B=4 L=2048 D=16"),
+    "c1": (8, 4096, 2048, "bfloat16", "bfloat16", 0.9, 0.1, 256, "bf16 B=8 L=4096 D=2048"),
+    "c2": (1, 65536, 4096, "float16", "float16", 0.99, 0.01, 1024, "fp16 B=1 L=65536 D=4096"),
+    "c3scan": (16, 2048, 4096, "float16", "float32", 0.9, 0.1, 256, "fp16 operands, fp32 y/dy, B=16 L=2048 D=4096"),
+    "c4scan": (32, 64, 1024, "float16", "float32", 0.9, 0.1, 256, "fp16 operands, fp32 y/dy, B=32 L=64 D=1024"),
+}
+
+
+def make_operands(torch, shape, dtype, out_dtype, a_lo, a_span, device, seed=0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    x = torch.randn(shape, generator=g)
+    a = torch.rand(shape, generator=g) * a_span + a_lo
+    b = torch.randn(shape, generator=g) * 0.1
+    c = torch.sigmoid(torch.randn(shape, generator=g))
+    dy = torch.randn(shape, generator=g)
+    ops = [t.to(dtype) for t in (x, a, b, c)] + [dy.to(out_dtype)]
+    return ops, [t.to(device) for t in ops]
+
+
+def event_time_ms(torch, fn, iters, warmup):
+    """Average duration of `fn` over `iters` back-to-back calls, from events on the current stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def cpu_baseline(torch, workload, shape, dtype, out_dtype, a_lo, a_span):
+    """The reference CPU path (torch restatement, oracle/reference_cpu_path.py) on a bounded slice."""
+    from oracle.reference_cpu_path import reference_scan_with_grads
+
+    B, L, D = shape
+    # one batch row keeps every time step and every column of the workload; very long rows are cut in time
+    sB, sL, sD = 1, min(L, 4096), D
+    ops, _ = make_operands(torch, (sB, sL, sD), dtype, out_dtype, a_lo, a_span, "cpu")
+    t0 = time.perf_counter()
+    reference_scan_with_grads(*ops, out_dtype=out_dtype)
+    dt = time.perf_counter() - t0
+    n = sB * sL * sD
+    es, os_ = ops[0].element_size(), ops[4].element_size()
+    nbytes = n * (8 * es + 2 * os_)
+    return {
+        "value": nbytes / dt / 1e9,
+        "unit": "GB/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"reference CPU path (python loop over batch and time, torch autograd backward) fwd+bwd on a "
+                  f"slice B={sB} L={sL} D={sD} of {workload}, {dt:.2f} s, host cpu_count={os.cpu_count()}",
+        "melem_per_s": n / dt / 1e6,
+        "seconds": dt,
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--tune-fwd", type=int, default=0, help="geometry override for sweeps (see qssm_plan_scan)")
+    ap.add_argument("--tune-bwd", type=int, default=0)
+    args = ap.parse_args()
+
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: rows (b, d) of the scan are independent, so more GPUs only shard B or D "
+              "with no communication. Run with --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from quick_ssm_amd import _lib, hip_scan
+    from quick_ssm_amd.scan_interface import scan
+
+    if not _lib.is_built():
+        from quick_ssm_amd import build as builder
+
+        builder.build(verbose=False)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the scan has no CPU product path to measure)", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+
+    B, L, D, dt_name, odt_name, a_lo, a_span, block_l, desc = WORKLOADS[args.workload]
+    dtype, out_dtype = getattr(torch, dt_name), getattr(torch, odt_name)
+    shape = (B, L, D)
+    n = B * L * D
+    cpu_ops, (x, a, b, c, dy) = make_operands(torch, shape, dtype, out_dtype, a_lo, a_span, dev)
+    del cpu_ops
+    es, os_ = x.element_size(), dy.element_size()
+    fwd_bytes = n * (4 * es + os_)
+    bwd_bytes = n * (8 * es + os_)
+    step_bytes = fwd_bytes + bwd_bytes
+
+    leaves = [t.requires_grad_(True) for t in (x, a, b, c)]
+
+    def step():
+        for t in leaves:
+            t.grad = None
+        y = scan(*leaves, block_l=block_l, checkpoint=True, out_dtype=out_dtype)
+        y.backward(dy)
+
+    # ---- whole step through the public API: W warm-ups, then exactly K timed steps ---------------
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(args.steps):
+        step()
+    ev1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    gpu_ms = ev0.elapsed_time(ev1) / args.steps
+    ms_per_step = wall_ms
+
+    # ---- the two kernels on their own, through the C ABI -------------------------------------------
+    xd, ad, bd, cd = (t.detach() for t in leaves)
+    with torch.no_grad():
+        _, _, ckpt, stride = hip_scan.scan_forward(xd, ad, bd, cd, out_dtype=out_dtype,
+                                                   tune=args.tune_fwd, bwd_tune=args.tune_bwd)
+        fwd_ms = event_time_ms(
+            torch, lambda: hip_scan.scan_forward(xd, ad, bd, cd, out_dtype=out_dtype, tune=args.tune_fwd,
+                                                 bwd_tune=args.tune_bwd), args.steps, args.warmup)
+        bwd_ms = event_time_ms(
+            torch, lambda: hip_scan.scan_backward(xd, ad, bd, cd, dy, ckpt=ckpt, ckpt_stride=stride,
+                                                  tune=args.tune_bwd), args.steps, args.warmup)
+        # achievable ceiling on this box: a plain copy of the same number of bytes as the backward moves
+        nb = (bwd_bytes // 2 // 16) * 16
+        src = torch.empty(nb, dtype=torch.uint8, device=dev)
+        dst = torch.empty(nb, dtype=torch.uint8, device=dev)
+        stream = torch.cuda.current_stream().cuda_stream
+        lib = _lib.load()
+        copy_ms = event_time_ms(torch, lambda: lib.qssm_copy_bytes(dst.data_ptr(), src.data_ptr(), nb, stream),
+                                args.steps, args.warmup)
+        del src, dst
+    status = hip_scan.workspace_status()
+    align = 4 if D % 4 == 0 else (2 if D % 2 == 0 else 1)
+    plan_b = hip_scan.make_plan(B, L, D, dtype, out_dtype, _lib.QSSM_BACKWARD, align, stride, args.tune_bwd)
+    plan_f = hip_scan.make_plan(B, L, D, dtype, out_dtype, _lib.QSSM_FORWARD, align, stride, args.tune_fwd)
+
+    traffic = None
+    traffic_file = ROOT / "profiles" / f"scan_bwd_{args.workload}_traffic.json"
+    if traffic_file.exists():
+        try:
+            traffic = json.loads(traffic_file.read_text()).get("traffic_bytes_per_launch")
+        except (ValueError, OSError):
+            traffic = None
+
+    bwd_gbs = bwd_bytes / (bwd_ms * 1e-3) / 1e9
+    fwd_gbs = fwd_bytes / (fwd_ms * 1e-3) / 1e9
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    out = {
+        "metric": "scan fwd+bwd HBM GB/s (% of peak) + Melem/s, bf16 B=8 L=4096 D=2048",
+        "value": value,
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {"float32": "f32", "float16": "f16", "bfloat16": "bf16"}[dt_name] + " storage, f32 arithmetic",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: gated linear scan fwd+bwd through scan(), {desc}, "
+                               f"block_l={block_l}, checkpoint=True", "B": B, "L": L, "D": D},
+        "pct_of_hbm_peak": 100.0 * value / HBM_PEAK_GBS,
+        "melem_per_s": n / (ms_per_step * 1e-3) / 1e6,
+        "algorithmic_bytes_per_step": step_bytes,
+        "gpu_ms_per_step_events": gpu_ms,
+        "kernels_only_gbs": step_bytes / ((fwd_ms + bwd_ms) * 1e-3) / 1e9,
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "scan_bwd_kernel",
+            "achieved": bwd_gbs,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": bwd_gbs / HBM_PEAK_GBS,
+            "traffic": traffic,
+            "algorithmic_bytes_per_launch": bwd_bytes,
+            "avg_launch_ms": bwd_ms,
+        },
+        "kernels": {
+            "scan_fwd_kernel": {"avg_launch_ms": fwd_ms, "algorithmic_bytes": fwd_bytes, "gbs": fwd_gbs,
+                                "frac": fwd_gbs / HBM_PEAK_GBS, "plan": plan_f.describe()},
+            "scan_bwd_kernel": {"avg_launch_ms": bwd_ms, "algorithmic_bytes": bwd_bytes, "gbs": bwd_gbs,
+                                "frac": bwd_gbs / HBM_PEAK_GBS, "plan": plan_b.describe()},
+            "copy_kernel": {"avg_launch_ms": copy_ms, "bytes_moved": 2 * nb, "gbs": 2 * nb / (copy_ms * 1e-3) / 1e9},
+        },
+        "workspace_status": status,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(torch, args.workload, shape, dtype, out_dtype, a_lo, a_span)
+    print(json.dumps(out), flush=True)
+    return 0 if status == 0 else 1
+
+
+if __name__ == "__main__":
+    sys.exit(main())

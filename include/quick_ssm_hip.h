@@ -23,7 +23,7 @@
  *   - Return value: 0 on success, a QSSM_E* code or a hipError_t (> 0) otherwise;
  *     qssm_error_string() describes the last failure on the calling thread.
  *   - Entry points are re-entrant.  Two launches that share one workspace must be ordered
- *     on one stream.
+ *     on one stream and carry different epochs.
  */
 #ifndef QUICK_SSM_HIP_H
 #define QUICK_SSM_HIP_H
@@ -61,8 +61,10 @@ extern "C" {
 /*
  * Launch geometry of one scan launch.  A "tile" is one workgroup's share: a strip of
  * `strip_cols` adjacent columns of one batch row, times `seg_len` consecutive time steps.
- * Tiles of one (batch, strip) chain hand a one-row carry to the next tile in time through the
- * workspace; `ckpt_stride` is the spacing of the fp32 states h(t-1) kept for the backward.
+ * Tiles of one (batch, strip) chain are grouped in clusters of `cluster` consecutive tiles; a
+ * tile reads the per-tile maps of its cluster through the workspace and one state per cluster
+ * is handed from cluster to cluster.  `ckpt_stride` is the spacing of the fp32 states h(t-1)
+ * kept for the backward.
  */
 typedef struct qssm_plan {
   int32_t B, L, D;
@@ -71,15 +73,19 @@ typedef struct qssm_plan {
   int32_t direction;      /* QSSM_FORWARD / QSSM_BACKWARD */
   int32_t vec;            /* adjacent columns per lane: 1, 2 or 4 */
   int32_t steps;          /* consecutive time steps per lane: 4 or 8 */
+  int32_t threads;        /* lanes per workgroup: 256, 512 or 1024 */
   int32_t g_log2;         /* log2(lanes per row of a strip) */
   int32_t strip_cols;     /* vec << g_log2 */
-  int32_t seg_len;        /* steps * (256 >> g_log2) */
+  int32_t seg_len;        /* steps * (threads >> g_log2) */
   int32_t n_strips;       /* ceil(D / strip_cols) */
   int32_t n_seg;          /* ceil(L / seg_len) */
+  int32_t cluster;        /* tiles per cluster (power of two) */
+  int32_t n_super;        /* ceil(n_seg / cluster) */
   int32_t ckpt_stride;    /* spacing (time steps) of saved states; divides seg_len */
   int32_t n_ckpt;         /* ceil(L / ckpt_stride) */
+  int32_t lds_bytes;      /* dynamic LDS per workgroup */
   int32_t reserved;
-  uint64_t workspace_bytes; /* carry workspace the launch needs (zero-filled, see below) */
+  uint64_t workspace_bytes; /* workspace the launch needs (see qssm_workspace_reset) */
   uint64_t ckpt_elems;      /* B * n_ckpt * D floats */
 } qssm_plan;
 
@@ -100,7 +106,9 @@ QSSM_API const char* qssm_error_string(void);
  *                 every base address expressed in elements, over all tensors of the launch.
  *   ckpt_stride : 0 lets the forward plan pick; a backward plan (and a forward plan that must
  *                 match one) passes the stride the saved states were written with.
- *   tune        : 0 = automatic; otherwise (g_log2 + 1) | (steps << 8) overrides for sweeps.
+ *   tune        : 0 = automatic; otherwise bit fields override single choices for sweeps, a zero field
+ *                 keeping the automatic one: (g_log2 + 1) | steps << 8 | max vec << 16 |
+ *                 threads code << 24 (1: 256, 2: 512, 3: 1024) | (log2(cluster) + 1) << 28.
  * Stands in for the grid/block arithmetic of block_scan_forward_3d
  * (quick_ssm/triton_forwards.py:157-167) and block_scan_backward_3d
  * (quick_ssm/triton_backwards.py:195-204).
@@ -110,9 +118,10 @@ QSSM_API int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, i
                    qssm_plan* plan);
 
 /*
- * Zero-fill a carry workspace (a fill kernel on `stream`, safe under graph capture).  A
- * workspace must be zero before its first launch; each launch leaves it zero again, so this is
- * needed once per allocation and after a launch that reported QSSM_ESTATE.
+ * Zero-fill a workspace (a fill kernel on `stream`, safe under graph capture).  A workspace
+ * must be zero before its first launch.  Launches mark what they write with their `epoch`, so
+ * the fill is needed once per allocation, again before an epoch value is ever reused, and after
+ * a launch that left a nonzero status.
  */
 QSSM_API int qssm_workspace_reset(void* workspace, uint64_t bytes, void* stream);
 
@@ -129,6 +138,8 @@ QSSM_API int qssm_workspace_status(const void* workspace, void* stream, int32_t*
  *   y          may be NULL (state-only pass: only `ckpt` is produced).
  *   h_out      optional fp32 [B, L, D] (strides sh): every h(t); the checkpoint=False case.
  *   ckpt       optional fp32 [B, n_ckpt, D] contiguous: h(t-1) at t = k * ckpt_stride.
+ *   epoch      nonzero, and different from the epoch of every earlier launch that used this
+ *              workspace since it was last zero-filled (a per-workspace counter does it).
  * Replaces _TritonScanFunction.forward's per-tile body (quick_ssm/scan_interface.py:91-107):
  * block_scan_forward_3d (quick_ssm/triton_forwards.py:134-172, three launches + fp32 scratch)
  * followed by y = c * h and the cast to out_dtype.
@@ -141,7 +152,7 @@ QSSM_API int qssm_scan_forward(const qssm_plan* plan,
                       void* y, qssm_strides sy,
                       float* h_out, qssm_strides sh,
                       float* ckpt,
-                      void* workspace, uint64_t workspace_bytes,
+                      void* workspace, uint64_t workspace_bytes, uint32_t epoch,
                       void* stream);
 
 /*
@@ -165,7 +176,7 @@ QSSM_API int qssm_scan_backward(const qssm_plan* plan,
                        void* da, qssm_strides sda,
                        void* db, qssm_strides sdb,
                        void* dc, qssm_strides sdc,
-                       void* workspace, uint64_t workspace_bytes,
+                       void* workspace, uint64_t workspace_bytes, uint32_t epoch,
                        void* stream);
 
 /*

@@ -42,13 +42,17 @@ class Plan(ctypes.Structure):
         ("direction", ctypes.c_int32),
         ("vec", ctypes.c_int32),
         ("steps", ctypes.c_int32),
+        ("threads", ctypes.c_int32),
         ("g_log2", ctypes.c_int32),
         ("strip_cols", ctypes.c_int32),
         ("seg_len", ctypes.c_int32),
         ("n_strips", ctypes.c_int32),
         ("n_seg", ctypes.c_int32),
+        ("cluster", ctypes.c_int32),
+        ("n_super", ctypes.c_int32),
         ("ckpt_stride", ctypes.c_int32),
         ("n_ckpt", ctypes.c_int32),
+        ("lds_bytes", ctypes.c_int32),
         ("reserved", ctypes.c_int32),
         ("workspace_bytes", ctypes.c_uint64),
         ("ckpt_elems", ctypes.c_uint64),
@@ -88,11 +92,11 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.qssm_workspace_status.argtypes = [vp, vp, ctypes.POINTER(i32)]
     lib.qssm_scan_forward.restype = ctypes.c_int
     lib.qssm_scan_forward.argtypes = (
-        [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, u64, vp]
+        [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, u64, ctypes.c_uint32, vp]
     )
     lib.qssm_scan_backward.restype = ctypes.c_int
     lib.qssm_scan_backward.argtypes = (
-        [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, Strides] * 4 + [vp, u64, vp]
+        [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, Strides] * 4 + [vp, u64, ctypes.c_uint32, vp]
     )
     lib.qssm_copy_bytes.restype = ctypes.c_int
     lib.qssm_copy_bytes.argtypes = [vp, vp, u64, vp]

@@ -38,10 +38,10 @@ static int pow2_ceil(int64_t n) {
   return p;
 }
 
-// Lanes that one row of D columns can feed at `vec` columns per lane (a power of two <= 256).
+// Lanes that one row of D columns can feed at `vec` columns per lane (a power of two <= 1024).
 static int lanes_cap(int D, int vec) {
   const int lanes = pow2_ceil(D > 0 ? (D + vec - 1) / vec : 1);
-  return lanes < kThreads ? lanes : kThreads;
+  return lanes < 1024 ? lanes : 1024;
 }
 
 static int ilog2(int n) {
@@ -77,21 +77,35 @@ static bool aligned_to(const void* p, int64_t sb, int64_t sl, int elem_bytes, in
   return (sb % vec == 0) && (sl % vec == 0);
 }
 
+static const int kMaxThreads = 1024;
+static const int kMaxLdsBytes = 64 * 1024;
+static const int kCUs = 256;
+
+static bool threads_ok(int t) { return t == 256 || t == 512 || t == 1024; }
+
 static int check_plan(const qssm_plan* pl, int direction) {
   if (pl == nullptr) return fail(QSSM_EINVAL, "plan is NULL");
   if (pl->direction != direction) return fail(QSSM_EINVAL, "plan was made for the other direction");
   if (pl->B < 0 || pl->L < 0 || pl->D < 0) return fail(QSSM_EINVAL, "negative dimension");
   if (pl->vec != 1 && pl->vec != 2 && pl->vec != 4) return fail(QSSM_EINVAL, "plan.vec must be 1, 2 or 4");
   if (pl->steps != 4 && pl->steps != 8) return fail(QSSM_EINVAL, "plan.steps must be 4 or 8");
-  if (pl->g_log2 < 0 || pl->g_log2 > 8) return fail(QSSM_EINVAL, "plan.g_log2 out of range");
+  if (!threads_ok(pl->threads)) return fail(QSSM_EINVAL, "plan.threads must be 256, 512 or 1024");
+  if (pl->g_log2 < 0 || (1 << pl->g_log2) > pl->threads) return fail(QSSM_EINVAL, "plan.g_log2 out of range");
   if (pl->D % pl->vec != 0) return fail(QSSM_EALIGN, "D=%d is not a multiple of plan.vec=%d", pl->D, pl->vec);
-  const int ng = kThreads >> pl->g_log2;
+  const int ng = pl->threads >> pl->g_log2;
   if (pl->strip_cols != (pl->vec << pl->g_log2) || pl->seg_len != pl->steps * ng)
     return fail(QSSM_EINVAL, "plan geometry is inconsistent");
   if (pl->B == 0 || pl->L == 0 || pl->D == 0) return 0;
   if (pl->n_strips != (pl->D + pl->strip_cols - 1) / pl->strip_cols ||
       pl->n_seg != (pl->L + pl->seg_len - 1) / pl->seg_len)
     return fail(QSSM_EINVAL, "plan tile counts are inconsistent");
+  if (pl->cluster < 1 || (pl->cluster & (pl->cluster - 1)) != 0 ||
+      pl->n_super != (pl->n_seg + pl->cluster - 1) / pl->cluster)
+    return fail(QSSM_EINVAL, "plan cluster counts are inconsistent");
+  const size_t lds = direction == QSSM_FORWARD ? fwd_lds_bytes(pl->threads, pl->vec, pl->strip_cols, pl->cluster)
+                                               : bwd_lds_bytes(pl->threads, pl->vec, pl->strip_cols, pl->cluster);
+  if ((size_t)pl->lds_bytes != lds || lds > (size_t)kMaxLdsBytes)
+    return fail(QSSM_EINVAL, "plan.lds_bytes=%d does not fit the geometry", pl->lds_bytes);
   // Forward lanes write a saved state only at their own first step; backward tiles read one
   // only at the tile's first step.
   if (pl->ckpt_stride <= 0 || pl->seg_len % pl->ckpt_stride != 0 ||
@@ -102,7 +116,15 @@ static int check_plan(const qssm_plan* pl, int direction) {
   return 0;
 }
 
-static void fill_geometry(Geometry* g, const qssm_plan* pl, void* workspace) {
+// Lane offsets inside a tile are 32-bit: the tile of every tensor must span less than 2 GiB.
+static bool tile_span_ok(const qssm_plan* pl, const void* p, int64_t sb, int64_t sl, int elem_bytes) {
+  if (p == nullptr) return true;
+  if (sl < 0 || sb < 0) return false;
+  const int64_t span = ((int64_t)pl->seg_len * sl + pl->strip_cols) * elem_bytes;
+  return span < ((int64_t)1 << 31);
+}
+
+static void fill_geometry(Geometry* g, const qssm_plan* pl, void* workspace, uint32_t epoch) {
   g->B = pl->B;
   g->L = pl->L;
   g->D = pl->D;
@@ -111,12 +133,17 @@ static void fill_geometry(Geometry* g, const qssm_plan* pl, void* workspace) {
   g->n_chains = pl->B * pl->n_strips;
   g->n_seg = pl->n_seg;
   g->seg_len = pl->seg_len;
+  g->cluster = pl->cluster;
+  g->n_super = pl->n_super;
   g->ckpt_stride = pl->ckpt_stride;
   g->n_ckpt = pl->n_ckpt;
+  g->epoch = epoch;
   char* ws = (char*)workspace;
   g->status = (int*)ws;
-  g->tickets = (unsigned*)(ws + kStatusBytes);
-  g->carry = (unsigned long long*)(ws + ws_carry_offset((uint64_t)g->n_chains));
+  g->tickets = (unsigned long long*)(ws + kStatusBytes);
+  g->maps = (unsigned long long*)(ws + ws_maps_offset((uint64_t)g->n_chains));
+  g->states = (unsigned long long*)(ws + ws_states_offset((uint64_t)g->n_chains, (uint64_t)g->n_seg,
+                                                          (uint64_t)pl->strip_cols));
 }
 
 }  // namespace qssm
@@ -153,52 +180,116 @@ int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int32_t ou
   // forward; the backward keeps 5 operands + h in registers, so fp32 stays at 8 bytes there.
   int vec = 4;
   if (es == 4 && direction == QSSM_BACKWARD) vec = 2;
+  const int tune_vec = (tune >> 16) & 0xff;
+  if (tune_vec == 1 || tune_vec == 2) vec = tune_vec < vec ? tune_vec : vec;
   while (vec > 1 && (align_elems % vec != 0 || (D > 0 && D % vec != 0))) vec >>= 1;
   plan->vec = vec;
 
-  // Steps per lane: 8 keeps chains short; the backward at 8 bytes per lane would not fit the
-  // register file at 8 steps.
+  // Steps per lane: 8 where the registers allow; the backward at 8 bytes per lane holds five
+  // operands plus h per step and stays at 4.
   int steps = 8;
   if (direction == QSSM_BACKWARD && vec * es >= 8) steps = 4;
+  const int tune_steps = (tune >> 8) & 0xff;
+  if (tune_steps == 4 || tune_steps == 8) steps = tune_steps;
 
-  // Lanes per row: 128-byte row pieces when D allows, never more lanes than the row has vectors.
+  // Lanes per row: 512-byte row pieces (what HBM needs to stream at full rate) when D allows,
+  // never more lanes than the row has vectors.  Workgroup: as many time groups as the sequence
+  // can feed, up to 1024 lanes, because every tile boundary along time costs a hand-over.
   const int cap = lanes_cap(D, vec);
-  int g = 128 / (vec * es);
-  if (g < 1) g = 1;
-  if (tune != 0) {
-    const int tg = (tune & 0xff) - 1, ts = (tune >> 8) & 0xff;
-    if (tg >= 0 && tg <= 8) g = 1 << tg;
-    if (ts == 4 || ts == 8) steps = ts;
-  } else {
-    // Short sequences: widen the rows rather than leave most time groups idle.
-    const int64_t lp2 = pow2_ceil(L > 0 ? L : 1);
-    while (g < cap && (int64_t)steps * (kThreads / g) / 2 >= lp2) g <<= 1;
-  }
+  int g = 512 / (vec * es);
   if (g > cap) g = cap;
+  int threads = kMaxThreads;
+  if (vec == 1) threads = 256;
+  const int tune_g = (tune & 0xff) - 1, tune_t = (tune >> 24) & 0xf;
+  const bool fixed_g = tune_g >= 0 && tune_g <= 10, fixed_t = tune_t >= 1 && tune_t <= 3;
+  if (fixed_g) g = 1 << tune_g;
+  if (fixed_t) threads = 256 << (tune_t - 1);
+  if (vec == 1 && threads != 256) threads = 256;
+  if (g > threads) g = threads;
+  auto tiles = [&](int gg, int tt) -> int64_t {
+    const int64_t strips = (D + (int64_t)gg * vec - 1) / ((int64_t)gg * vec);
+    const int64_t seg = (int64_t)steps * (tt / gg);
+    return (int64_t)B * strips * ((L + seg - 1) / seg);
+  };
+  if (B > 0 && L > 0 && D > 0) {
+    const int64_t lp2 = pow2_ceil(L);
+    // A tile longer than the sequence only idles lanes: shed time groups first.
+    auto fit_threads = [&]() {
+      if (!fixed_t)
+        while (threads > 256 && threads / 2 >= g && (int64_t)steps * (threads / 2 / g) >= lp2) threads >>= 1;
+    };
+    fit_threads();
+    // Small problems: rather more workgroups than idle compute units.  Narrow the strips first
+    // (more chains, no extra hand-overs), then cut the tiles shorter in time.
+    if (!fixed_g) {
+      while (g * vec * es > 128 && g > 1 && tiles(g, threads) < 2 * kCUs) {
+        g >>= 1;
+        fit_threads();
+      }
+    }
+    if (!fixed_t)
+      while (threads > 256 && threads / 2 >= g && tiles(g, threads) < 2 * kCUs) threads >>= 1;
+    // Very short sequences: widen the rows instead of idling most time groups of a workgroup.
+    if (!fixed_g)
+      while (g < cap && g < threads && (int64_t)steps * (threads / g) / 2 >= lp2) g <<= 1;
+  }
   if (ckpt_stride > 0) {
-    // A tile must cover a whole number of saved-state intervals and a lane must not straddle one.
+    // A tile must cover a whole number of saved-state intervals and a forward lane must not
+    // straddle one.
     if ((ckpt_stride & (ckpt_stride - 1)) != 0 || ckpt_stride < 4)
       return fail(QSSM_EINVAL, "ckpt_stride=%d must be a power of two >= 4", ckpt_stride);
     if (direction == QSSM_FORWARD && ckpt_stride % steps != 0) steps = 4;
-    while (steps * (kThreads / g) < ckpt_stride && g > 1) g >>= 1;
-    if ((steps * (kThreads / g)) % ckpt_stride != 0)
+    while (steps * (threads / g) < ckpt_stride && threads < kMaxThreads && vec > 1) threads <<= 1;
+    while (steps * (threads / g) < ckpt_stride && g > 1) g >>= 1;
+    if ((steps * (threads / g)) % ckpt_stride != 0)
       return fail(QSSM_EINVAL, "ckpt_stride=%d does not fit any tile length", ckpt_stride);
   }
+  // Wide workgroups exist for vec >= 2 only, and the 1024-lane backward at 4 columns per lane
+  // only at 4 steps (register file).
+  if (direction == QSSM_BACKWARD && vec == 4 && steps == 8 && threads == 1024) threads = 512;
+  if (g > threads) g = threads;
   plan->steps = steps;
+  plan->threads = threads;
   plan->g_log2 = ilog2(g);
   plan->strip_cols = vec << plan->g_log2;
-  plan->seg_len = steps * (kThreads >> plan->g_log2);
+  plan->seg_len = steps * (threads >> plan->g_log2);
   if (ckpt_stride > 0 && plan->seg_len % ckpt_stride != 0)
     return fail(QSSM_EINVAL, "ckpt_stride=%d does not divide seg_len=%d", ckpt_stride, plan->seg_len);
   plan->ckpt_stride = ckpt_stride > 0 ? ckpt_stride : plan->seg_len;
-  if (B == 0 || L == 0 || D == 0) return 0;
+  plan->cluster = 1;
+  if (B == 0 || L == 0 || D == 0) {
+    plan->lds_bytes = (int32_t)(direction == QSSM_FORWARD ? fwd_lds_bytes(threads, vec, plan->strip_cols, 1)
+                                                          : bwd_lds_bytes(threads, vec, plan->strip_cols, 1));
+    return 0;
+  }
   plan->n_strips = (D + plan->strip_cols - 1) / plan->strip_cols;
   plan->n_seg = (L + plan->seg_len - 1) / plan->seg_len;
   plan->n_ckpt = (L + plan->ckpt_stride - 1) / plan->ckpt_stride;
+
+  // Cluster size: each cluster boundary is one serial hand-over (about 1.3 us under load on
+  // MI355X); keep their number per chain at 32 or fewer when LDS allows.
+  int cluster = 1;
+  const int tune_r = (tune >> 28) & 0xf;
+  if (tune_r >= 1) {
+    cluster = 1 << (tune_r - 1);
+  } else {
+    while (cluster < 8 && (plan->n_seg + cluster - 1) / cluster > 32) cluster <<= 1;
+  }
+  auto lds_for = [&](int r) -> size_t {
+    return direction == QSSM_FORWARD ? fwd_lds_bytes(threads, vec, plan->strip_cols, r)
+                                     : bwd_lds_bytes(threads, vec, plan->strip_cols, r);
+  };
+  while (cluster > 1 && lds_for(cluster) > (size_t)kMaxLdsBytes) cluster >>= 1;
+  if (lds_for(cluster) > (size_t)kMaxLdsBytes) return fail(QSSM_EINVAL, "geometry needs too much LDS");
+  plan->cluster = cluster;
+  plan->n_super = (plan->n_seg + cluster - 1) / cluster;
+  plan->lds_bytes = (int32_t)lds_for(cluster);
+
   const uint64_t n_chains = (uint64_t)B * plan->n_strips;
   if (n_chains * plan->n_seg > 0x7fffffffull) return fail(QSSM_EINVAL, "shape needs more than 2^31 tiles");
-  plan->workspace_bytes =
-      ws_carry_offset(n_chains) + (plan->n_seg > 1 ? n_chains * plan->n_seg * plan->strip_cols * 8ull : 0ull);
+  plan->workspace_bytes = plan->n_seg > 1 ? ws_total_bytes(n_chains, (uint64_t)plan->n_seg, (uint64_t)plan->n_super,
+                                                           (uint64_t)plan->strip_cols)
+                                          : ws_maps_offset(n_chains);
   plan->ckpt_elems = (uint64_t)B * plan->n_ckpt * D;
   return 0;
 }
@@ -227,7 +318,7 @@ int qssm_workspace_status(const void* workspace, void* stream, int32_t* status) 
 int qssm_scan_forward(const qssm_plan* plan, const void* x, qssm_strides sx, const void* a, qssm_strides sa,
                       const void* b, qssm_strides sb, const void* c, qssm_strides sc, void* y, qssm_strides sy,
                       float* h_out, qssm_strides sh, float* ckpt, void* workspace, uint64_t workspace_bytes,
-                      void* stream) {
+                      uint32_t epoch, void* stream) {
   int rc = check_plan(plan, QSSM_FORWARD);
   if (rc != 0) return rc;
   if (plan->B == 0 || plan->L == 0 || plan->D == 0) return 0;
@@ -244,14 +335,21 @@ int qssm_scan_forward(const qssm_plan* plan, const void* x, qssm_strides sx, con
     return fail(QSSM_EWORKSPACE, "workspace has %llu bytes, plan needs %llu", (unsigned long long)workspace_bytes,
                 (unsigned long long)plan->workspace_bytes);
 
+  if (epoch == 0) return fail(QSSM_EINVAL, "epoch must be nonzero");
+  if (!tile_span_ok(plan, x, sx.b, sx.l, es) || !tile_span_ok(plan, a, sa.b, sa.l, es) ||
+      !tile_span_ok(plan, b, sb.b, sb.l, es) || !tile_span_ok(plan, c, sc.b, sc.l, es) ||
+      !tile_span_ok(plan, y, sy.b, sy.l, os) || !tile_span_ok(plan, h_out, sh.b, sh.l, 4))
+    return fail(QSSM_EINVAL, "a time stride is negative or too large for 32-bit tile offsets; pass a contiguous copy");
+
   FwdArgs args;
-  fill_geometry(&args.g, plan, workspace);
+  fill_geometry(&args.g, plan, workspace, epoch);
   args.x = x; args.a = a; args.b = b; args.c = c; args.y = y; args.h_out = h_out; args.ckpt = ckpt;
   args.x_sb = sx.b; args.x_sl = sx.l; args.a_sb = sa.b; args.a_sl = sa.l;
   args.b_sb = sb.b; args.b_sl = sb.l; args.c_sb = sc.b; args.c_sl = sc.l;
   args.y_sb = sy.b; args.y_sl = sy.l; args.h_sb = sh.b; args.h_sl = sh.l;
   const dim3 grid((unsigned)((uint64_t)args.g.n_chains * args.g.n_seg));
-  fn(args, plan->vec, plan->steps, grid, (hipStream_t)stream);
+  if (!fn(args, plan->vec, plan->steps, plan->threads, grid, (size_t)plan->lds_bytes, (hipStream_t)stream))
+    return fail(QSSM_EINVAL, "no forward kernel for vec=%d steps=%d threads=%d", plan->vec, plan->steps, plan->threads);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : hip_fail(e, "scan_fwd_kernel launch");
 }
@@ -260,7 +358,8 @@ int qssm_scan_backward(const qssm_plan* plan, const void* x, qssm_strides sx, co
                        const void* b, qssm_strides sb, const void* c, qssm_strides sc, const void* dy,
                        qssm_strides sdy, const float* h, qssm_strides sh, const float* ckpt, void* dx,
                        qssm_strides sdx, void* da, qssm_strides sda, void* db, qssm_strides sdb, void* dc,
-                       qssm_strides sdc, void* workspace, uint64_t workspace_bytes, void* stream) {
+                       qssm_strides sdc, void* workspace, uint64_t workspace_bytes, uint32_t epoch,
+                       void* stream) {
   int rc = check_plan(plan, QSSM_BACKWARD);
   if (rc != 0) return rc;
   if (plan->B == 0 || plan->L == 0 || plan->D == 0) return 0;
@@ -280,8 +379,16 @@ int qssm_scan_backward(const qssm_plan* plan, const void* x, qssm_strides sx, co
     return fail(QSSM_EWORKSPACE, "workspace has %llu bytes, plan needs %llu", (unsigned long long)workspace_bytes,
                 (unsigned long long)plan->workspace_bytes);
 
+  if (epoch == 0) return fail(QSSM_EINVAL, "epoch must be nonzero");
+  if (!tile_span_ok(plan, x, sx.b, sx.l, es) || !tile_span_ok(plan, a, sa.b, sa.l, es) ||
+      !tile_span_ok(plan, b, sb.b, sb.l, es) || !tile_span_ok(plan, c, sc.b, sc.l, es) ||
+      !tile_span_ok(plan, dy, sdy.b, sdy.l, os) || !tile_span_ok(plan, dx, sdx.b, sdx.l, es) ||
+      !tile_span_ok(plan, da, sda.b, sda.l, es) || !tile_span_ok(plan, db, sdb.b, sdb.l, es) ||
+      !tile_span_ok(plan, dc, sdc.b, sdc.l, es))
+    return fail(QSSM_EINVAL, "a time stride is negative or too large for 32-bit tile offsets; pass a contiguous copy");
+
   BwdArgs args;
-  fill_geometry(&args.g, plan, workspace);
+  fill_geometry(&args.g, plan, workspace, epoch);
   args.x = x; args.a = a; args.b = b; args.c = c; args.dy = dy; args.h = h; args.ckpt = ckpt;
   args.dx = dx; args.da = da; args.db = db; args.dc = dc;
   args.x_sb = sx.b; args.x_sl = sx.l; args.a_sb = sa.b; args.a_sl = sa.l;
@@ -290,7 +397,8 @@ int qssm_scan_backward(const qssm_plan* plan, const void* x, qssm_strides sx, co
   args.dx_sb = sdx.b; args.dx_sl = sdx.l; args.da_sb = sda.b; args.da_sl = sda.l;
   args.db_sb = sdb.b; args.db_sl = sdb.l; args.dc_sb = sdc.b; args.dc_sl = sdc.l;
   const dim3 grid((unsigned)((uint64_t)args.g.n_chains * args.g.n_seg));
-  fn(args, plan->vec, plan->steps, grid, (hipStream_t)stream);
+  if (!fn(args, plan->vec, plan->steps, plan->threads, grid, (size_t)plan->lds_bytes, (hipStream_t)stream))
+    return fail(QSSM_EINVAL, "no backward kernel for vec=%d steps=%d threads=%d", plan->vec, plan->steps, plan->threads);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : hip_fail(e, "scan_bwd_kernel launch");
 }

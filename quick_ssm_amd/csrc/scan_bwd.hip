@@ -20,25 +20,32 @@
 
 namespace qssm {
 
-template <typename Tin, typename Tout, int VEC, int T>
-__global__ void __launch_bounds__(kThreads) scan_bwd_kernel(const BwdArgs p) {
-  __shared__ float sA[kThreads * VEC];
-  __shared__ float sXf[kThreads * VEC];
-  __shared__ float sXe[kThreads * VEC];
-  __shared__ float sEin[kThreads * VEC];
-  __shared__ int sSeg;
-
+template <typename Tin, typename Tout, int VEC, int T, int NTH>
+__global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
+  extern __shared__ float lds[];
   const Geometry& g = p.g;
+  const int G = 1 << g.g_log2;
+  const int NG = NTH >> g.g_log2;
+  const int cols = G * VEC;
+  const int R = g.cluster;
+  float* sA = lds;                       // [NTH * VEC] per-lane map, multiplier (both directions)
+  float* sXf = sA + NTH * VEC;           // [NTH * VEC] forward offset
+  float* sXe = sXf + NTH * VEC;          // [NTH * VEC] reverse offset
+  float* sPA = sXe + NTH * VEC;          // [(R-1) * cols] reverse maps of the later tiles of the cluster
+  float* sPX = sPA + (R - 1) * cols;
+  float* sE = sPX + (R - 1) * cols;      // [cols] reverse carry entering the tile
+  int* sSeg = reinterpret_cast<int*>(sE + cols);
+
   const int tid = threadIdx.x;
   const int chain = blockIdx.x % g.n_chains;
 
   // ---- claim a tile of this chain, last tile in time first -----------------------------------
   int seg = 0;
   if (g.n_seg > 1) {
-    if (tid == 0) sSeg = (int)claim_ticket(g.tickets, chain, g.n_seg);
+    if (tid == 0) *sSeg = (int)claim_ticket(g.tickets, chain, g.epoch);
     __syncthreads();
-    const int tk = sSeg;
-    if (tk >= g.n_seg) {  // workspace was not zero on entry
+    const int tk = __builtin_amdgcn_readfirstlane(*sSeg);
+    if ((unsigned)tk >= (unsigned)g.n_seg) {  // more claims than tiles: the epoch was reused
       if (tid == 0) raise_status(g.status, 2);
       return;
     }
@@ -47,60 +54,63 @@ __global__ void __launch_bounds__(kThreads) scan_bwd_kernel(const BwdArgs p) {
 
   const int bi = chain / g.n_strips;
   const int strip = chain - bi * g.n_strips;
-  const int G = 1 << g.g_log2;
-  const int NG = kThreads >> g.g_log2;
   const int j = tid >> g.g_log2;
   const int dl = (tid & (G - 1)) * VEC;
-  const int cols = G * VEC;
   const int d = strip * cols + dl;
   const bool dok = d < g.D;
   const int t_tile = seg * g.seg_len;
   const int t0 = t_tile + j * T;
   const bool have_h = p.h != nullptr;
 
-  const Tin* xp = (const Tin*)p.x + (int64_t)bi * p.x_sb + (int64_t)t0 * p.x_sl + d;
-  const Tin* ap = (const Tin*)p.a + (int64_t)bi * p.a_sb + (int64_t)t0 * p.a_sl + d;
-  const Tin* bp = (const Tin*)p.b + (int64_t)bi * p.b_sb + (int64_t)t0 * p.b_sl + d;
-  const Tin* cp = (const Tin*)p.c + (int64_t)bi * p.c_sb + (int64_t)t0 * p.c_sl + d;
-  const Tout* gp = (const Tout*)p.dy + (int64_t)bi * p.dy_sb + (int64_t)t0 * p.dy_sl + d;
+  const int64_t col0 = (int64_t)strip * cols;
+  const char* xb = (const char*)p.x + ((int64_t)bi * p.x_sb + (int64_t)t_tile * p.x_sl + col0) * (int64_t)sizeof(Tin);
+  const char* ab = (const char*)p.a + ((int64_t)bi * p.a_sb + (int64_t)t_tile * p.a_sl + col0) * (int64_t)sizeof(Tin);
+  const char* bb = (const char*)p.b + ((int64_t)bi * p.b_sb + (int64_t)t_tile * p.b_sl + col0) * (int64_t)sizeof(Tin);
+  const char* cb = (const char*)p.c + ((int64_t)bi * p.c_sb + (int64_t)t_tile * p.c_sl + col0) * (int64_t)sizeof(Tin);
+  const char* gb = (const char*)p.dy + ((int64_t)bi * p.dy_sb + (int64_t)t_tile * p.dy_sl + col0) * (int64_t)sizeof(Tout);
+  const uint32_t xo = (uint32_t)((j * T * (int)p.x_sl + dl) * (int)sizeof(Tin)), xs = (uint32_t)p.x_sl * sizeof(Tin);
+  const uint32_t ao = (uint32_t)((j * T * (int)p.a_sl + dl) * (int)sizeof(Tin)), as = (uint32_t)p.a_sl * sizeof(Tin);
+  const uint32_t bo = (uint32_t)((j * T * (int)p.b_sl + dl) * (int)sizeof(Tin)), bs = (uint32_t)p.b_sl * sizeof(Tin);
+  const uint32_t co = (uint32_t)((j * T * (int)p.c_sl + dl) * (int)sizeof(Tin)), cs = (uint32_t)p.c_sl * sizeof(Tin);
+  const uint32_t go = (uint32_t)((j * T * (int)p.dy_sl + dl) * (int)sizeof(Tout)), gs = (uint32_t)p.dy_sl * sizeof(Tout);
   const float* hp = p.h + (int64_t)bi * p.h_sb + (int64_t)t0 * p.h_sl + d;
 
   // ---- issue every load of the tile before touching any of them ------------------------------
-  Pack<Tin, VEC> rx[T], ra[T], rb[T], rc[T];
-  Pack<Tout, VEC> rg[T];
+  Words<Tin, VEC> rx[T], ra[T], rb[T], rc[T];
+  Words<Tout, VEC> rg[T];
   float hs[T][VEC];   // h(t0 + i)
-  float hprev[VEC];   // h(t0 - 1), then the tile-level state for the rebuild
+  float hprev[VEC];   // h(t0 - 1); before the rebuild, the state at the tile's first step
   const bool tile_full = (t_tile + g.seg_len <= g.L) && ((strip + 1) * cols <= g.D);
   if (tile_full) {
 #pragma unroll
     for (int i = 0; i < T; ++i) {
-      ra[i] = load_pack<Tin, VEC>(ap + (int64_t)i * p.a_sl);
-      rc[i] = load_pack<Tin, VEC>(cp + (int64_t)i * p.c_sl);
-      rg[i] = load_pack<Tout, VEC>(gp + (int64_t)i * p.dy_sl);
+      ra[i] = load_stream<Tin, VEC>(ab, ao + i * as);
+      rc[i] = load_stream<Tin, VEC>(cb, co + i * cs);
+      rg[i] = load_stream<Tout, VEC>(gb, go + i * gs);
     }
 #pragma unroll
     for (int i = 0; i < T; ++i) {
-      rb[i] = load_pack<Tin, VEC>(bp + (int64_t)i * p.b_sl);
-      rx[i] = load_pack<Tin, VEC>(xp + (int64_t)i * p.x_sl);
+      rb[i] = load_stream<Tin, VEC>(bb, bo + i * bs);
+      rx[i] = load_stream<Tin, VEC>(xb, xo + i * xs);
     }
   } else {
     // Steps past L and columns past D act as the identity map (a = 1, everything else 0).
 #pragma unroll
     for (int i = 0; i < T; ++i) {
-      ra[i] = fill_pack<Tin, VEC>(1.0f);
-      rb[i] = fill_pack<Tin, VEC>(0.0f);
-      rx[i] = fill_pack<Tin, VEC>(0.0f);
-      rc[i] = fill_pack<Tin, VEC>(0.0f);
-      rg[i] = fill_pack<Tout, VEC>(0.0f);
+      ra[i] = fill_words<Tin, VEC>(true);
+      rb[i] = fill_words<Tin, VEC>(false);
+      rx[i] = fill_words<Tin, VEC>(false);
+      rc[i] = fill_words<Tin, VEC>(false);
+      rg[i] = fill_words<Tout, VEC>(false);
     }
 #pragma unroll
     for (int i = 0; i < T; ++i) {
       if (dok && t0 + i < g.L) {
-        ra[i] = load_pack<Tin, VEC>(ap + (int64_t)i * p.a_sl);
-        rc[i] = load_pack<Tin, VEC>(cp + (int64_t)i * p.c_sl);
-        rg[i] = load_pack<Tout, VEC>(gp + (int64_t)i * p.dy_sl);
-        rb[i] = load_pack<Tin, VEC>(bp + (int64_t)i * p.b_sl);
-        rx[i] = load_pack<Tin, VEC>(xp + (int64_t)i * p.x_sl);
+        ra[i] = load_stream<Tin, VEC>(ab, ao + i * as);
+        rc[i] = load_stream<Tin, VEC>(cb, co + i * cs);
+        rg[i] = load_stream<Tout, VEC>(gb, go + i * gs);
+        rb[i] = load_stream<Tin, VEC>(bb, bo + i * bs);
+        rx[i] = load_stream<Tin, VEC>(xb, xo + i * xs);
       }
     }
   }
@@ -138,16 +148,18 @@ __global__ void __launch_bounds__(kThreads) scan_bwd_kernel(const BwdArgs p) {
   for (int i = 0; i < T; ++i) {
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
-      const float av = to_f32(ra[i].v[v]);
-      Xf[v] = av * Xf[v] + to_f32(rb[i].v[v]) * to_f32(rx[i].v[v]);
+      const float av = elem(ra[i], v);
+      Xf[v] = av * Xf[v] + elem(rb[i], v) * elem(rx[i], v);
       A[v] = av * A[v];
     }
+    __builtin_amdgcn_sched_barrier(0);
   }
 #pragma unroll
   for (int i = T - 1; i >= 0; --i) {
 #pragma unroll
     for (int v = 0; v < VEC; ++v)
-      Xe[v] = to_f32(ra[i].v[v]) * (to_f32(rc[i].v[v]) * to_f32(rg[i].v[v]) + Xe[v]);
+      Xe[v] = elem(ra[i], v) * (elem(rc[i], v) * elem(rg[i], v) + Xe[v]);
+    __builtin_amdgcn_sched_barrier(0);
   }
 #pragma unroll
   for (int v = 0; v < VEC; ++v) {
@@ -155,6 +167,8 @@ __global__ void __launch_bounds__(kThreads) scan_bwd_kernel(const BwdArgs p) {
     sXf[tid * VEC + v] = Xf[v];
     sXe[tid * VEC + v] = Xe[v];
   }
+#pragma unroll
+  for (int i = 0; i < T; ++i) { forget(ra[i]); forget(rb[i]); forget(rx[i]); forget(rc[i]); forget(rg[i]); }
   __syncthreads();
 
   // ---- compose: groups before this one (forward state), groups after it (reverse carry) --------
@@ -180,28 +194,72 @@ __global__ void __launch_bounds__(kThreads) scan_bwd_kernel(const BwdArgs p) {
     }
   }
 
-  // ---- chain: the first lane group owns the tile's total reverse map ---------------------------
-  if (j == 0) {
-    unsigned long long* cw = g.carry + ((int64_t)chain * g.n_seg + seg) * cols + dl;
+  // ---- reverse carry entering the tile -----------------------------------------------------------
+  float ein[VEC];
 #pragma unroll
-    for (int v = 0; v < VEC; ++v) {
-      float ein = 0.0f;
-      if (dok) {
-        if (seg + 1 < g.n_seg && !carry_consume(cw + cols + v, &ein)) raise_status(g.status, 1);
-        if (seg > 0) {
-          const float atot = A[v] * As[v];
-          const float xtot = A[v] * Xs[v] + Xe[v];
-          carry_publish(cw + v, atot * ein + xtot);
+  for (int v = 0; v < VEC; ++v) ein[v] = 0.0f;
+  if (g.n_seg > 1) {
+    const int s = seg / R;                                     // cluster of this tile
+    const int m = seg - s * R;                                 // tiles of the cluster before this one
+    const int last = ((s + 1) * R < g.n_seg ? (s + 1) * R : g.n_seg) - 1;
+    const int cnt = last - seg;                                // tiles of the cluster after this one
+    const bool edge = (j == 0);  // the first lane group holds the tile's total reverse map
+    float At[VEC], Xt[VEC];
+    if (edge) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) { At[v] = A[v] * As[v]; Xt[v] = A[v] * Xs[v] + Xe[v]; }
+      // Earlier tiles of the cluster need this tile's map; it depends on nothing, so it goes out first.
+      if (dok && m > 0) {
+        unsigned long long* mw = g.maps + (((int64_t)chain * g.n_seg + seg) * cols + dl) * 2;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          word_publish(mw + 2 * v, g.epoch, At[v]);
+          word_publish(mw + 2 * v + 1, g.epoch, Xt[v]);
         }
       }
-      sEin[dl + v] = ein;
     }
+    if (cnt > 0) {
+      // Lane group j fetches the maps of the later tiles seg+1+j, seg+1+j+NG, ... of the cluster.
+      for (int i = j; i < cnt; i += NG) {
+        if (dok) {
+          float w[2 * VEC];
+          const unsigned long long* mw = g.maps + (((int64_t)chain * g.n_seg + (seg + 1 + i)) * cols + dl) * 2;
+          if (!words_wait<2 * VEC>(mw, g.epoch, w)) raise_status(g.status, 1);
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) {
+            sPA[i * cols + dl + v] = w[2 * v];
+            sPX[i * cols + dl + v] = w[2 * v + 1];
+          }
+        }
+      }
+      __syncthreads();
+    }
+    if (edge) {
+      // The one serial hop: the carry the next cluster in time hands back.
+      if (dok && s + 1 < g.n_super) {
+        const unsigned long long* sw = g.states + ((int64_t)chain * g.n_super + (s + 1)) * cols + dl;
+        if (!words_wait<VEC>(sw, g.epoch, ein)) raise_status(g.status, 1);
+      }
+      for (int i = cnt - 1; i >= 0; --i) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) ein[v] = sPA[i * cols + dl + v] * ein[v] + sPX[i * cols + dl + v];
+      }
+      if (dok && m == 0 && s > 0) {
+        unsigned long long* sw = g.states + ((int64_t)chain * g.n_super + s) * cols + dl;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) word_publish(sw + v, g.epoch, At[v] * ein[v] + Xt[v]);
+      }
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) sE[dl + v] = ein[v];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) ein[v] = sE[dl + v];
   }
-  __syncthreads();
 
   float E[VEC];
 #pragma unroll
-  for (int v = 0; v < VEC; ++v) E[v] = As[v] * sEin[dl + v] + Xs[v];
+  for (int v = 0; v < VEC; ++v) E[v] = As[v] * ein[v] + Xs[v];
 
   // ---- sweep 2: rebuild h over this lane's steps -------------------------------------------------
   if (!have_h) {
@@ -212,53 +270,69 @@ __global__ void __launch_bounds__(kThreads) scan_bwd_kernel(const BwdArgs p) {
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
         const float hm = (i == 0) ? hprev[v] : hs[i - 1][v];
-        hs[i][v] = to_f32(ra[i].v[v]) * hm + to_f32(rb[i].v[v]) * to_f32(rx[i].v[v]);
+        hs[i][v] = elem(ra[i], v) * hm + elem(rb[i], v) * elem(rx[i], v);
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 
   // ---- sweep 3: reverse recurrence and the four gradients ---------------------------------------
-  Tin* dxp = (Tin*)p.dx + (int64_t)bi * p.dx_sb + (int64_t)t0 * p.dx_sl + d;
-  Tin* dap = (Tin*)p.da + (int64_t)bi * p.da_sb + (int64_t)t0 * p.da_sl + d;
-  Tin* dbp = (Tin*)p.db + (int64_t)bi * p.db_sb + (int64_t)t0 * p.db_sl + d;
-  Tin* dcp = (Tin*)p.dc + (int64_t)bi * p.dc_sb + (int64_t)t0 * p.dc_sl + d;
+  char* dxb = (char*)p.dx + ((int64_t)bi * p.dx_sb + (int64_t)t_tile * p.dx_sl + col0) * (int64_t)sizeof(Tin);
+  char* dab = (char*)p.da + ((int64_t)bi * p.da_sb + (int64_t)t_tile * p.da_sl + col0) * (int64_t)sizeof(Tin);
+  char* dbb = (char*)p.db + ((int64_t)bi * p.db_sb + (int64_t)t_tile * p.db_sl + col0) * (int64_t)sizeof(Tin);
+  char* dcb = (char*)p.dc + ((int64_t)bi * p.dc_sb + (int64_t)t_tile * p.dc_sl + col0) * (int64_t)sizeof(Tin);
+  const uint32_t dxo = (uint32_t)((j * T * (int)p.dx_sl + dl) * (int)sizeof(Tin)), dxs = (uint32_t)p.dx_sl * sizeof(Tin);
+  const uint32_t dao = (uint32_t)((j * T * (int)p.da_sl + dl) * (int)sizeof(Tin)), das = (uint32_t)p.da_sl * sizeof(Tin);
+  const uint32_t dbo = (uint32_t)((j * T * (int)p.db_sl + dl) * (int)sizeof(Tin)), dbs = (uint32_t)p.db_sl * sizeof(Tin);
+  const uint32_t dco = (uint32_t)((j * T * (int)p.dc_sl + dl) * (int)sizeof(Tin)), dcs = (uint32_t)p.dc_sl * sizeof(Tin);
 #pragma unroll
   for (int i = T - 1; i >= 0; --i) {
-    Pack<Tin, VEC> vdx, vda, vdb, vdc;
+    float vdx[VEC], vda[VEC], vdb[VEC], vdc[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
-      const float gy = to_f32(rg[i].v[v]);
-      const float dH = to_f32(rc[i].v[v]) * gy + E[v];
+      const float gy = elem(rg[i], v);
+      const float dH = elem(rc[i], v) * gy + E[v];
       const float hm = (i == 0) ? hprev[v] : hs[i - 1][v];
-      vdc.v[v] = (Tin)(gy * hs[i][v]);
-      vdx.v[v] = (Tin)(to_f32(rb[i].v[v]) * dH);
-      vdb.v[v] = (Tin)(to_f32(rx[i].v[v]) * dH);
-      vda.v[v] = (Tin)(hm * dH);
-      E[v] = to_f32(ra[i].v[v]) * dH;
+      vdc[v] = gy * hs[i][v];
+      vdx[v] = elem(rb[i], v) * dH;
+      vdb[v] = elem(rx[i], v) * dH;
+      vda[v] = hm * dH;
+      E[v] = elem(ra[i], v) * dH;
     }
     if (tile_full || (dok && t0 + i < g.L)) {
-      if (p.dx != nullptr) store_pack<Tin, VEC>(dxp + (int64_t)i * p.dx_sl, vdx);
-      if (p.da != nullptr) store_pack<Tin, VEC>(dap + (int64_t)i * p.da_sl, vda);
-      if (p.db != nullptr) store_pack<Tin, VEC>(dbp + (int64_t)i * p.db_sl, vdb);
-      if (p.dc != nullptr) store_pack<Tin, VEC>(dcp + (int64_t)i * p.dc_sl, vdc);
+      if (p.dx != nullptr) store_stream<Tin, VEC>(dxb, dxo + i * dxs, vdx);
+      if (p.da != nullptr) store_stream<Tin, VEC>(dab, dao + i * das, vda);
+      if (p.db != nullptr) store_stream<Tin, VEC>(dbb, dbo + i * dbs, vdb);
+      if (p.dc != nullptr) store_stream<Tin, VEC>(dcb, dco + i * dcs, vdc);
     }
+    // Keep each step's conversions next to their use (register footprint).
+    __builtin_amdgcn_sched_barrier(0);
   }
 }
 
 template <typename Tin, typename Tout>
-static void launch_bwd(const BwdArgs& args, int vec, int steps, dim3 grid, hipStream_t stream) {
-#define QSSM_BWD_CASE(V, S)                                                              \
-  if (vec == V && steps == S) {                                                          \
-    hipLaunchKernelGGL((scan_bwd_kernel<Tin, Tout, V, S>), grid, dim3(kThreads), 0, stream, args); \
-    return;                                                                              \
+static bool launch_bwd(const BwdArgs& args, int vec, int steps, int threads, dim3 grid, size_t lds,
+                       hipStream_t stream) {
+#define QSSM_BWD_CASE(V, S, N)                                                                        \
+  if (vec == V && steps == S && threads == N) {                                                       \
+    hipLaunchKernelGGL((scan_bwd_kernel<Tin, Tout, V, S, N>), grid, dim3(N), lds, stream, args);       \
+    return true;                                                                                      \
   }
-  QSSM_BWD_CASE(1, 4)
-  QSSM_BWD_CASE(1, 8)
-  QSSM_BWD_CASE(2, 4)
-  QSSM_BWD_CASE(2, 8)
-  QSSM_BWD_CASE(4, 4)
-  QSSM_BWD_CASE(4, 8)
+  QSSM_BWD_CASE(1, 4, 256)
+  QSSM_BWD_CASE(1, 8, 256)
+  QSSM_BWD_CASE(2, 4, 256)
+  QSSM_BWD_CASE(2, 8, 256)
+  QSSM_BWD_CASE(4, 4, 256)
+  QSSM_BWD_CASE(4, 8, 256)
+  QSSM_BWD_CASE(2, 4, 512)
+  QSSM_BWD_CASE(2, 8, 512)
+  QSSM_BWD_CASE(4, 4, 512)
+  QSSM_BWD_CASE(4, 8, 512)
+  QSSM_BWD_CASE(2, 4, 1024)
+  QSSM_BWD_CASE(2, 8, 1024)
+  QSSM_BWD_CASE(4, 4, 1024)
 #undef QSSM_BWD_CASE
+  return false;
 }
 
 bwd_launch_fn find_bwd_launcher(int in_dtype, int out_dtype) {

@@ -1,21 +1,29 @@
 // Shared device-side pieces of the gfx950 gated linear scan kernels.
 //
-// Tile model (both directions).  A workgroup of 256 lanes owns one tile: a strip of
-// `G * VEC` adjacent columns of one batch row, times `seg_len = NG * T` consecutive time
-// steps, where G = lanes per row (a power of two, runtime), NG = 256 / G lane groups, and each
-// lane keeps T steps x VEC columns of every operand in registers.  Lanes of one group read one
-// contiguous row piece (G * VEC * sizeof(elem) bytes, 128 B at the default geometry), so all
-// global traffic is coalesced along D while the recurrence runs along L inside a lane.
+// Tile model (both directions).  A workgroup of NTH lanes owns one tile: a strip of `G * VEC`
+// adjacent columns of one batch row, times `seg_len = NG * T` consecutive time steps, where
+// G = lanes per row (a power of two, runtime), NG = NTH / G lane groups, and each lane keeps
+// T steps x VEC columns of every operand in registers.  Lanes of one group read one contiguous
+// row piece (G * VEC * sizeof(elem) bytes; 512 B at the default geometry, which is what HBM
+// needs to stream at full rate), so all global traffic is coalesced along D while the
+// recurrence runs along L inside a lane.
 //
 //   sweep 1   every lane folds its T steps into one affine map (A, X) starting from identity
 //   LDS       the NG maps of each column are exchanged; lane group j composes the maps of the
 //             groups before it (forward) / after it (reverse) into its carry-in
-//   chain     the tile-level carry comes from the neighbouring tile of the same chain through
-//             a 64-bit {flag, fp32} word in the workspace (one word per column)
+//   chain     tiles of one (batch row, strip) chain are grouped in clusters of R consecutive
+//             tiles.  A tile publishes its own affine map as soon as it has it (it depends on
+//             nothing), reads the maps of the tiles before it in its cluster, and takes the
+//             state at the cluster's edge from the previous cluster.  Only that last hand-over
+//             is a serial dependency: one hop per cluster, not per tile.
 //   sweep 2   every lane re-runs its T steps from the true carry-in and stores the results
 //
-// Tiles of a chain are claimed in time order through a per-chain ticket counter, so the tile a
-// workgroup waits for was always claimed by a workgroup that is already running.
+// Words exchanged between workgroups are {epoch:32 | fp32 bits:32}: flag and payload travel
+// in one 64-bit access, so no fence is needed between them, and a word left over from an
+// earlier launch (older epoch) reads as "not there yet".  Agent scope makes the accesses
+// coherent across the XCDs' separate L2 caches.  Tiles of a chain are claimed in time order
+// through a per-chain ticket counter (also epoch-tagged), so every tile a workgroup waits for
+// was claimed by a workgroup that is already running.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -25,19 +33,26 @@
 
 namespace qssm {
 
-constexpr int kThreads = 256;
-// Polls before a tile gives up on its neighbour's carry (each poll sleeps ~64 clocks and costs
-// a round trip to the coherent level of the memory system: about a second in total).
+// Polls before a tile gives up on a neighbour's word (each poll is a round trip to the
+// coherent level of the memory system plus a short sleep: roughly a second in total).
 constexpr int kSpinLimit = 1 << 20;
 
-// Workspace layout (bytes): [0,64) status word; then one 64-byte slot per chain holding its
-// ticket counter; then, 256-byte aligned, n_chains * n_seg * strip_cols carry words of 8 bytes.
+// Workspace layout (bytes): [0,64) status word; one 64-byte slot per chain holding its ticket
+// counter; then, 256-byte aligned, the tile maps (2 words per column per tile); then the
+// cluster states (1 word per column per cluster).
 constexpr uint64_t kStatusBytes = 64;
 constexpr uint64_t kTicketStride = 64;
 
-__host__ __device__ inline uint64_t ws_carry_offset(uint64_t n_chains) {
-  uint64_t off = kStatusBytes + n_chains * kTicketStride;
-  return (off + 255u) & ~uint64_t(255);
+__host__ __device__ inline uint64_t ws_align(uint64_t off) { return (off + 255u) & ~uint64_t(255); }
+__host__ __device__ inline uint64_t ws_maps_offset(uint64_t n_chains) {
+  return ws_align(kStatusBytes + n_chains * kTicketStride);
+}
+__host__ __device__ inline uint64_t ws_states_offset(uint64_t n_chains, uint64_t n_seg, uint64_t cols) {
+  return ws_align(ws_maps_offset(n_chains) + n_chains * n_seg * cols * 16u);
+}
+__host__ __device__ inline uint64_t ws_total_bytes(uint64_t n_chains, uint64_t n_seg, uint64_t n_super,
+                                                   uint64_t cols) {
+  return ws_align(ws_states_offset(n_chains, n_seg, cols) + n_chains * n_super * cols * 8u);
 }
 
 typedef _Float16 f16_t;
@@ -54,7 +69,113 @@ template <> struct RawOf<4> { typedef unsigned int type; };
 template <> struct RawOf<8> { typedef unsigned int type __attribute__((ext_vector_type(2))); };
 template <> struct RawOf<16> { typedef unsigned int type __attribute__((ext_vector_type(4))); };
 
-// One vector load / store of VEC elements (the pointer is VEC-element aligned by contract).
+// VEC stored elements of one operand at one time step, kept as the 32-bit words they were
+// loaded as.  16-bit elements stay packed two to a register until the instruction that uses
+// them (a struct of halves would be split into one register per element).
+template <typename T, int V>
+struct Words {
+  static constexpr int N = (int)((sizeof(T) * V + 3) / 4);
+  uint32_t w[N];
+};
+
+template <typename T> struct ElemBits;
+template <> struct ElemBits<float> {
+  static __device__ __forceinline__ uint32_t one() { return 0x3f800000u; }
+  template <int V> static __device__ __forceinline__ float get(const Words<float, V>& p, int v) {
+    return __uint_as_float(p.w[v]);
+  }
+  template <int V> static __device__ __forceinline__ void set(Words<float, V>& p, const float* f) {
+#pragma unroll
+    for (int v = 0; v < V; ++v) p.w[v] = __float_as_uint(f[v]);
+  }
+};
+template <> struct ElemBits<bf16_t> {
+  static __device__ __forceinline__ uint32_t one() { return 0x3f803f80u; }
+  template <int V> static __device__ __forceinline__ float get(const Words<bf16_t, V>& p, int v) {
+    const uint32_t w = p.w[v >> 1];
+    return __uint_as_float((v & 1) ? (w & 0xffff0000u) : (w << 16));
+  }
+  template <int V> static __device__ __forceinline__ void set(Words<bf16_t, V>& p, const float* f) {
+    if (V == 1) {
+      p.w[0] = (uint32_t)__builtin_bit_cast(unsigned short, (bf16_t)f[0]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < V / 2; ++k) {
+        const uint32_t lo = __builtin_bit_cast(unsigned short, (bf16_t)f[2 * k]);
+        const uint32_t hi = __builtin_bit_cast(unsigned short, (bf16_t)f[2 * k + 1]);
+        p.w[k] = lo | (hi << 16);
+      }
+    }
+  }
+};
+template <> struct ElemBits<f16_t> {
+  static __device__ __forceinline__ uint32_t one() { return 0x3c003c00u; }
+  template <int V> static __device__ __forceinline__ float get(const Words<f16_t, V>& p, int v) {
+    const uint32_t w = p.w[v >> 1];
+    const unsigned short h = (unsigned short)((v & 1) ? (w >> 16) : (w & 0xffffu));
+    return (float)__builtin_bit_cast(f16_t, h);
+  }
+  template <int V> static __device__ __forceinline__ void set(Words<f16_t, V>& p, const float* f) {
+    if (V == 1) {
+      p.w[0] = (uint32_t)__builtin_bit_cast(unsigned short, (f16_t)f[0]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < V / 2; ++k) {
+        const uint32_t lo = __builtin_bit_cast(unsigned short, (f16_t)f[2 * k]);
+        const uint32_t hi = __builtin_bit_cast(unsigned short, (f16_t)f[2 * k + 1]);
+        p.w[k] = lo | (hi << 16);
+      }
+    }
+  }
+};
+
+template <typename T, int V>
+__device__ __forceinline__ float elem(const Words<T, V>& p, int v) {
+  return ElemBits<T>::template get<V>(p, v);
+}
+
+// One vector load / store of VEC elements at a byte offset from a workgroup-uniform base.
+// Operands and results are touched exactly once, so they are marked non-temporal (streaming).
+template <typename T, int V>
+__device__ __forceinline__ Words<T, V> load_stream(const char* base, uint32_t byte_off) {
+  typedef typename RawOf<sizeof(T) * V>::type raw_t;
+  const raw_t r = __builtin_nontemporal_load(reinterpret_cast<const raw_t*>(base + byte_off));
+  Words<T, V> out;
+  if constexpr (sizeof(T) * V <= 4) {
+    out.w[0] = (uint32_t)r;
+  } else {
+#pragma unroll
+    for (int k = 0; k < Words<T, V>::N; ++k) out.w[k] = r[k];
+  }
+  return out;
+}
+
+template <typename T, int V>
+__device__ __forceinline__ void store_stream(char* base, uint32_t byte_off, const float* f) {
+  typedef typename RawOf<sizeof(T) * V>::type raw_t;
+  Words<T, V> p;
+  ElemBits<T>::template set<V>(p, f);
+  raw_t r;
+  if constexpr (sizeof(T) * V <= 4) {
+    r = (raw_t)p.w[0];
+  } else {
+#pragma unroll
+    for (int k = 0; k < Words<T, V>::N; ++k) r[k] = p.w[k];
+  }
+  __builtin_nontemporal_store(r, reinterpret_cast<raw_t*>(base + byte_off));
+}
+
+// All VEC elements equal to 1 (`one`) or 0.
+template <typename T, int V>
+__device__ __forceinline__ Words<T, V> fill_words(bool one) {
+  Words<T, V> p;
+  uint32_t w = one ? ElemBits<T>::one() : 0u;
+  if (sizeof(T) * V < 4) w &= 0xffffu;
+#pragma unroll
+  for (int k = 0; k < Words<T, V>::N; ++k) p.w[k] = w;
+  return p;
+}
+
 template <typename T, int V>
 __device__ __forceinline__ Pack<T, V> load_pack(const T* p) {
   typedef typename RawOf<sizeof(T) * V>::type raw_t;
@@ -68,56 +189,60 @@ __device__ __forceinline__ void store_pack(T* p, const Pack<T, V>& v) {
   *reinterpret_cast<raw_t*>(p) = __builtin_bit_cast(raw_t, v);
 }
 
+// Makes the compiler forget what it knows about a loaded operand, so that the later sweeps
+// convert it to fp32 again instead of keeping an fp32 copy of every operand alive across the
+// barriers (which would double the register footprint of a tile).
 template <typename T, int V>
-__device__ __forceinline__ Pack<T, V> fill_pack(float f) {
-  Pack<T, V> r;
+__device__ __forceinline__ void forget(Words<T, V>& p) {
 #pragma unroll
-  for (int v = 0; v < V; ++v) r.v[v] = (T)f;
-  return r;
+  for (int k = 0; k < Words<T, V>::N; ++k) asm volatile("" : "+v"(p.w[k]));
 }
 
-__device__ __forceinline__ float to_f32(float v) { return v; }
-__device__ __forceinline__ float to_f32(f16_t v) { return (float)v; }
-__device__ __forceinline__ float to_f32(bf16_t v) { return (float)v; }
+// ---- words exchanged between workgroups ------------------------------------------------------
 
-// ---- cross-workgroup carry words ------------------------------------------------------------
-// A carry word is {flag:32 | fp32 bits:32}.  Flag and payload travel in one 64-bit access, so
-// no fence is needed between them; agent scope makes the access coherent across the XCDs'
-// separate L2 caches.
-
-constexpr unsigned kFlagReady = 1u;
-
-__device__ __forceinline__ void carry_publish(unsigned long long* w, float v) {
-  unsigned long long word = ((unsigned long long)kFlagReady << 32) | (unsigned long long)__float_as_uint(v);
+__device__ __forceinline__ void word_publish(unsigned long long* w, unsigned epoch, float v) {
+  const unsigned long long word = ((unsigned long long)epoch << 32) | (unsigned long long)__float_as_uint(v);
   __hip_atomic_store(w, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Wait for a published word, take its payload and leave the word zero for the next launch.
-// Returns false (and a NaN payload) if the neighbour never published within kSpinLimit polls.
-__device__ __forceinline__ bool carry_consume(unsigned long long* w, float* out) {
-  int spins = 0;
-  for (;;) {
-    unsigned long long word = __hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if ((unsigned)(word >> 32) == kFlagReady) {
-      *out = __uint_as_float((unsigned)word);
-      __hip_atomic_store(w, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// Wait until N consecutive words carry this launch's epoch; all N loads of a round are in
+// flight together.  Returns false (and NaN payloads) if they never all arrive.
+template <int N>
+__device__ __forceinline__ bool words_wait(const unsigned long long* w, unsigned epoch, float* out) {
+  for (int spins = 0; spins < kSpinLimit; ++spins) {
+    unsigned long long r[N];
+#pragma unroll
+    for (int n = 0; n < N; ++n)
+      r[n] = __hip_atomic_load(const_cast<unsigned long long*>(w) + n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    bool ok = true;
+#pragma unroll
+    for (int n = 0; n < N; ++n) ok = ok && ((unsigned)(r[n] >> 32) == epoch);
+    if (ok) {
+#pragma unroll
+      for (int n = 0; n < N; ++n) out[n] = __uint_as_float((unsigned)r[n]);
       return true;
-    }
-    if (++spins >= kSpinLimit) {
-      *out = __uint_as_float(0x7fc00000u);
-      return false;
     }
     __builtin_amdgcn_s_sleep(1);
   }
+#pragma unroll
+  for (int n = 0; n < N; ++n) out[n] = __uint_as_float(0x7fc00000u);
+  return false;
 }
 
-// Claim the next tile of `chain` in time order.  The holder of the last ticket puts the
-// counter back to zero: by then every other tile of the chain has taken its ticket.
-__device__ __forceinline__ unsigned claim_ticket(unsigned* tickets, int chain, int n_seg) {
-  unsigned* slot = tickets + (size_t)chain * (kTicketStride / sizeof(unsigned));
-  unsigned tk = __hip_atomic_fetch_add(slot, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  if (tk == (unsigned)(n_seg - 1)) __hip_atomic_store(slot, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  return tk;
+// Claim the next tile of `chain` in time order.  A ticket slot is {epoch:32 | count:32} like
+// every other word of the workspace: a slot that still carries another launch's epoch (or
+// anything else an earlier launch with a different layout left there) counts as zero, so the
+// workspace never has to be put back in order between launches.
+__device__ __forceinline__ unsigned claim_ticket(unsigned long long* tickets, int chain, unsigned epoch) {
+  unsigned long long* slot = tickets + (size_t)chain * (kTicketStride / sizeof(unsigned long long));
+  unsigned long long old = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  for (;;) {
+    const bool mine = (unsigned)(old >> 32) == epoch;
+    const unsigned long long next = mine ? old + 1ull : (((unsigned long long)epoch << 32) | 1ull);
+    if (__hip_atomic_compare_exchange_strong(slot, &old, next, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT))
+      return mine ? (unsigned)old : 0u;
+  }
 }
 
 __device__ __forceinline__ void raise_status(int* status, int code) {
@@ -133,11 +258,15 @@ struct Geometry {
   int n_chains;     // B * n_strips
   int n_seg;        // tiles per chain
   int seg_len;      // time steps per tile
+  int cluster;      // tiles per cluster (R, power of two)
+  int n_super;      // clusters per chain
   int ckpt_stride;  // spacing of saved states
   int n_ckpt;       // saved states per (batch, column)
+  unsigned epoch;   // this launch's flag value (nonzero)
   int* status;
-  unsigned* tickets;
-  unsigned long long* carry;
+  unsigned long long* tickets;
+  unsigned long long* maps;    // [chain][tile][col][2]: the tile's affine map (A, X)
+  unsigned long long* states;  // [chain][cluster][col]: state handed to the next cluster
 };
 
 struct FwdArgs {
@@ -159,9 +288,20 @@ struct BwdArgs {
   int64_t dx_sb, dx_sl, da_sb, da_sl, db_sb, db_sl, dc_sb, dc_sl;
 };
 
+// Dynamic LDS a launch needs: per-lane maps plus the cluster's neighbour maps and one row of state.
+inline size_t fwd_lds_bytes(int nth, int vec, int cols, int cluster) {
+  return sizeof(float) * ((size_t)2 * nth * vec + (size_t)2 * (cluster - 1) * cols + cols) + 16;
+}
+inline size_t bwd_lds_bytes(int nth, int vec, int cols, int cluster) {
+  return sizeof(float) * ((size_t)3 * nth * vec + (size_t)2 * (cluster - 1) * cols + cols) + 16;
+}
+
 // Host-side launch tables, one entry per (in dtype, out dtype) pair the library instantiates.
-typedef void (*fwd_launch_fn)(const FwdArgs&, int vec, int steps, dim3 grid, hipStream_t stream);
-typedef void (*bwd_launch_fn)(const BwdArgs&, int vec, int steps, dim3 grid, hipStream_t stream);
+// Return false if (vec, steps, threads) is not an instantiated combination.
+typedef bool (*fwd_launch_fn)(const FwdArgs&, int vec, int steps, int threads, dim3 grid, size_t lds,
+                              hipStream_t stream);
+typedef bool (*bwd_launch_fn)(const BwdArgs&, int vec, int steps, int threads, dim3 grid, size_t lds,
+                              hipStream_t stream);
 
 fwd_launch_fn find_fwd_launcher(int in_dtype, int out_dtype);
 bwd_launch_fn find_bwd_launcher(int in_dtype, int out_dtype);

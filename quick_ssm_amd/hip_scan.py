@@ -28,7 +28,9 @@ _BUILT_OUT = {
 }
 
 _ws_lock = threading.Lock()
-_workspaces: Dict[Tuple[int, int], Tensor] = {}
+# (device index, stream handle) -> [workspace tensor, last epoch used on it]
+_workspaces: Dict[Tuple[int, int], list] = {}
+_EPOCH_MAX = 0xFFFFFFFF
 
 
 def kernel_dtypes(in_dtypes: Sequence[torch.dtype], out_dtype: torch.dtype) -> Tuple[torch.dtype, torch.dtype]:
@@ -81,20 +83,23 @@ def _align_elems(tensors: Sequence[Optional[Tensor]], D: int) -> int:
     return 1
 
 
-def _workspace(device: torch.device, stream: int, nbytes: int) -> Tensor:
-    """Zero-initialised carry workspace for (device, stream), grown on demand.
+def _workspace(device: torch.device, stream: int, nbytes: int) -> Tuple[Tensor, int]:
+    """Workspace for (device, stream), grown on demand, and the epoch for the next launch on it.
 
-    A launch leaves its workspace zero again, so the buffer is filled once, at allocation
-    (torch.zeros runs a fill kernel on the current stream, ahead of the launch that uses it).
+    A workspace is zero-filled when it is allocated (torch.zeros runs a fill kernel on the current
+    stream, ahead of the launch that uses it).  Every launch then gets the next epoch value, so words
+    written by earlier launches never look valid; when the 32-bit counter is used up the buffer is
+    replaced by a fresh zeroed one.
     """
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
     with _ws_lock:
-        ws = _workspaces.get(key)
-        if ws is None or ws.numel() < nbytes:
+        entry = _workspaces.get(key)
+        if entry is None or entry[0].numel() < nbytes or entry[1] >= _EPOCH_MAX:
             size = max(1 << 20, 1 << (int(nbytes) - 1).bit_length())
-            ws = torch.zeros(size, dtype=torch.uint8, device=device)
-            _workspaces[key] = ws
-        return ws
+            entry = [torch.zeros(size, dtype=torch.uint8, device=device), 0]
+            _workspaces[key] = entry
+        entry[1] += 1
+        return entry[0], entry[1]
 
 
 def workspace_status(device: Optional[torch.device] = None) -> int:
@@ -103,9 +108,10 @@ def workspace_status(device: Optional[torch.device] = None) -> int:
     stream = torch.cuda.current_stream(device).cuda_stream
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
     with _ws_lock:
-        ws = _workspaces.get(key)
-    if ws is None:
+        entry = _workspaces.get(key)
+    if entry is None:
         return 0
+    ws = entry[0]
     out = ctypes.c_int32(0)
     _lib.check(_lib.load().qssm_workspace_status(ws.data_ptr(), stream, ctypes.byref(out)))
     return int(out.value)
@@ -176,13 +182,13 @@ def scan_forward(
 
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
-        ws = _workspace(dev, stream, int(plan.workspace_bytes))
+        ws, epoch = _workspace(dev, stream, int(plan.workspace_bytes))
         _lib.check(
             _lib.load().qssm_scan_forward(
                 ctypes.byref(plan),
                 _ptr(x), _strides(x), _ptr(a), _strides(a), _ptr(b), _strides(b), _ptr(c), _strides(c),
                 _ptr(y), _strides(y), _ptr(h), _strides(h), _ptr(ckpt),
-                ws.data_ptr(), ws.numel(), stream,
+                ws.data_ptr(), ws.numel(), epoch, stream,
             )
         )
     return y, h, ckpt, int(plan.ckpt_stride)
@@ -222,7 +228,7 @@ def scan_backward(
 
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
-        ws = _workspace(dev, stream, int(plan.workspace_bytes))
+        ws, epoch = _workspace(dev, stream, int(plan.workspace_bytes))
         _lib.check(
             _lib.load().qssm_scan_backward(
                 ctypes.byref(plan),
@@ -230,7 +236,7 @@ def scan_backward(
                 _ptr(dy), _strides(dy), _ptr(h), _strides(h), _ptr(ckpt),
                 _ptr(grads[0]), _strides(grads[0]), _ptr(grads[1]), _strides(grads[1]),
                 _ptr(grads[2]), _strides(grads[2]), _ptr(grads[3]), _strides(grads[3]),
-                ws.data_ptr(), ws.numel(), stream,
+                ws.data_ptr(), ws.numel(), epoch, stream,
             )
         )
     return tuple(grads)

@@ -19,7 +19,7 @@ def test_library_exports_every_declared_symbol(hip_lib):
     for name in declared:
         assert getattr(hip_lib, name) is not None
     assert hip_lib.qssm_version() == 100
-    assert ctypes.sizeof(_lib.Plan) == 16 * 4 + 2 * 8
+    assert ctypes.sizeof(_lib.Plan) == 20 * 4 + 2 * 8
 
 
 def test_chunk_ranges_follow_the_reference_rules():
@@ -48,7 +48,8 @@ def test_plans_are_consistent_and_forward_follows_backward(hip_lib, shape, dtype
         for p in (bwd, fwd):
             assert D % p.vec == 0 and p.vec <= align
             assert p.strip_cols == p.vec << p.g_log2
-            assert p.seg_len == p.steps * (256 >> p.g_log2)
+            assert p.threads in (256, 512, 1024) and p.seg_len == p.steps * (p.threads >> p.g_log2)
+            assert p.n_super == -(-p.n_seg // p.cluster) and 0 < p.lds_bytes <= 64 * 1024
             assert p.n_strips * p.strip_cols >= D > (p.n_strips - 1) * p.strip_cols
             assert p.n_seg * p.seg_len >= L > (p.n_seg - 1) * p.seg_len
             assert p.seg_len % p.ckpt_stride == 0
@@ -79,9 +80,9 @@ def test_plan_rejects_bad_arguments(hip_lib):
 def test_launchers_validate_before_touching_the_gpu(hip_lib):
     plan = hip_scan.make_plan(2, 64, 8, torch.float32, torch.float32, _lib.QSSM_FORWARD, 4)
     z = _lib.Strides(0, 0)
-    args = [ctypes.byref(plan)] + [None, z] * 6 + [None, None, 0, None]
+    args = [ctypes.byref(plan)] + [None, z] * 6 + [None, None, 0, 1, None]
     assert hip_lib.qssm_scan_forward(*args) == _lib.QSSM_EINVAL      # NULL operands
-    bwd = [ctypes.byref(plan)] + [None, z] * 6 + [None] + [None, z] * 4 + [None, 0, None]
+    bwd = [ctypes.byref(plan)] + [None, z] * 6 + [None] + [None, z] * 4 + [None, 0, 1, None]
     assert hip_lib.qssm_scan_backward(*bwd) == _lib.QSSM_EINVAL      # forward plan given to the backward
     assert b"direction" in hip_lib.qssm_error_string()
     assert hip_lib.qssm_copy_bytes(8, 16, 10, None) == _lib.QSSM_EALIGN
@@ -145,3 +146,56 @@ def test_ssm_layer_on_cpu_matches_hand_written_recurrence():
     assert [n for n, _ in layer.named_parameters()] == [
         "A_proj.weight", "A_proj.bias", "B_proj.weight", "C_proj_a.weight", "C_proj_b.weight", "D_proj.weight",
         "out_proj.weight", "out_proj.bias", "pre_norm.weight"]
+
+
+def _tile_accesses(plan, B, L, D):
+    """Element offsets (contiguous [B, L, D]) every lane of every tile touches, and the workspace words,
+    following the index arithmetic of the kernels."""
+    import numpy as np
+
+    G = 1 << plan.g_log2
+    NG = plan.threads >> plan.g_log2
+    cols = plan.strip_cols
+    tid = np.arange(plan.threads)
+    j, dl = tid >> plan.g_log2, (tid & (G - 1)) * plan.vec
+    n_chains = B * plan.n_strips
+    hi_elem, hi_ckpt, hi_word = -1, -1, -1
+    lo_elem = 0
+    maps_off = (64 + n_chains * 64 + 255) // 256 * 256
+    states_off = (maps_off + n_chains * plan.n_seg * cols * 16 + 255) // 256 * 256
+    for chain in range(n_chains):
+        bi, strip = divmod(chain, plan.n_strips)
+        d = strip * cols + dl
+        dok = d < D
+        for seg in range(plan.n_seg):
+            t0 = seg * plan.seg_len + j * plan.steps
+            for i in range(plan.steps):
+                ok = dok & (t0 + i < L)
+                if ok.any():
+                    off = (bi * L + t0[ok] + i) * D + d[ok]
+                    lo_elem = min(lo_elem, int(off.min()))
+                    hi_elem = max(hi_elem, int(off.max()) + plan.vec - 1)
+            ck = dok & (t0 < L) & (t0 % plan.ckpt_stride == 0)
+            if ck.any():
+                hi_ckpt = max(hi_ckpt, int(((bi * plan.n_ckpt + t0[ck] // plan.ckpt_stride) * D + d[ck]).max()) + plan.vec - 1)
+            if plan.n_seg > 1:
+                edge = dl[dok]
+                hi_word = max(hi_word, maps_off + int((((chain * plan.n_seg + seg) * cols + edge) * 2).max() + 2 * plan.vec) * 8)
+                s = seg // plan.cluster
+                hi_word = max(hi_word, states_off + int(((chain * plan.n_super + s) * cols + edge).max() + plan.vec) * 8)
+    assert NG * plan.steps == plan.seg_len
+    return lo_elem, hi_elem, hi_ckpt, hi_word
+
+
+@pytest.mark.parametrize("shape", [(2, 1500, 260), (2, 300, 5), (3, 7, 2), (2, 777, 64), (1, 2100, 520), (2, 64, 1024)],
+                         ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_tile_index_arithmetic_stays_in_bounds(hip_lib, shape, dtype):
+    B, L, D = shape
+    for direction in (_lib.QSSM_BACKWARD, _lib.QSSM_FORWARD):
+        for tune in (0, 1 | (4 << 8) | (1 << 24) | (2 << 28), 7 | (8 << 8) | (2 << 24) | (4 << 28)):
+            plan = hip_scan.make_plan(B, L, D, dtype, dtype, direction, 4, 0, tune)
+            lo, hi, hi_ckpt, hi_word = _tile_accesses(plan, B, L, D)
+            assert lo >= 0 and hi == B * L * D - 1          # every element is covered, nothing beyond
+            assert hi_ckpt < plan.ckpt_elems
+            assert hi_word <= plan.workspace_bytes
