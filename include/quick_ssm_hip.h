@@ -22,8 +22,7 @@
  *   - Arithmetic is fp32 whatever the storage type; y and the gradients are rounded once.
  *   - Return value: 0 on success, a QSSM_E* code or a hipError_t (> 0) otherwise;
  *     qssm_error_string() describes the last failure on the calling thread.
- *   - Entry points are re-entrant.  Two launches that share one workspace must be ordered
- *     on one stream and carry different epochs.
+ *   - Entry points are re-entrant (no global state).
  */
 #ifndef QUICK_SSM_HIP_H
 #define QUICK_SSM_HIP_H
@@ -85,7 +84,8 @@ typedef struct qssm_plan {
   int32_t n_ckpt;         /* ceil(L / ckpt_stride) */
   int32_t lds_bytes;      /* dynamic LDS per workgroup */
   int32_t reserved;
-  uint64_t workspace_bytes; /* workspace the launch needs (see qssm_workspace_reset) */
+  uint64_t control_bytes;   /* control block the launch needs (status word + ticket counters) */
+  uint64_t workspace_bytes; /* workspace the launch needs (words exchanged between workgroups) */
   uint64_t ckpt_elems;      /* B * n_ckpt * D floats */
 } qssm_plan;
 
@@ -118,19 +118,26 @@ QSSM_API int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, i
                    qssm_plan* plan);
 
 /*
- * Zero-fill a workspace (a fill kernel on `stream`, safe under graph capture).  A workspace
- * must be zero before its first launch.  Launches mark what they write with their `epoch`, so
- * the fill is needed once per allocation, again before an epoch value is ever reused, and after
- * a launch that left a nonzero status.
+ * Two device buffers accompany every launch, both owned by the caller and both zero-filled
+ * (qssm_zero_fill) when they are allocated:
+ *
+ *   control    status word + one ticket counter per chain (plan.control_bytes).  A launch needs it
+ *              zero on entry and leaves it zero, except that the status word becomes nonzero if
+ *              a tile gave up waiting for a neighbour (the outputs of that launch are then
+ *              poisoned with NaN and the buffer must be zero-filled again).
+ *   workspace  the words tiles hand to each other (plan.workspace_bytes; may be 0).  Words are
+ *              tagged with the launch's `epoch`, so nothing has to be cleared between launches:
+ *              zero-fill it once, and again before an epoch value would be reused.
+ *
+ * Launches that share these buffers must be ordered on one stream and carry different epochs.
  */
-QSSM_API int qssm_workspace_reset(void* workspace, uint64_t bytes, void* stream);
 
-/*
- * Read back the status word of a workspace (synchronises `stream`).  0 = every launch since
- * the last reset completed; nonzero = a tile gave up waiting for its neighbour's carry and
- * the outputs of that launch are poisoned with NaN.
- */
-QSSM_API int qssm_workspace_status(const void* workspace, void* stream, int32_t* status);
+/* Zero-fill a buffer with a fill kernel on `stream` (safe under graph capture; no hipMemset). */
+QSSM_API int qssm_zero_fill(void* buffer, uint64_t bytes, void* stream);
+
+/* Read back the status word of a control block (synchronises `stream`).  0 = every launch since
+ * the last zero-fill completed. */
+QSSM_API int qssm_control_status(const void* control, void* stream, int32_t* status);
 
 /*
  * Forward scan: one pass that reads x, a, b, c once and writes y once.
@@ -140,6 +147,7 @@ QSSM_API int qssm_workspace_status(const void* workspace, void* stream, int32_t*
  *   ckpt       optional fp32 [B, n_ckpt, D] contiguous: h(t-1) at t = k * ckpt_stride.
  *   epoch      nonzero, and different from the epoch of every earlier launch that used this
  *              workspace since it was last zero-filled (a per-workspace counter does it).
+ *   control, workspace: see above.
  * Replaces _TritonScanFunction.forward's per-tile body (quick_ssm/scan_interface.py:91-107):
  * block_scan_forward_3d (quick_ssm/triton_forwards.py:134-172, three launches + fp32 scratch)
  * followed by y = c * h and the cast to out_dtype.
@@ -152,6 +160,7 @@ QSSM_API int qssm_scan_forward(const qssm_plan* plan,
                       void* y, qssm_strides sy,
                       float* h_out, qssm_strides sh,
                       float* ckpt,
+                      void* control, uint64_t control_size,
                       void* workspace, uint64_t workspace_bytes, uint32_t epoch,
                       void* stream);
 
@@ -176,6 +185,7 @@ QSSM_API int qssm_scan_backward(const qssm_plan* plan,
                        void* da, qssm_strides sda,
                        void* db, qssm_strides sdb,
                        void* dc, qssm_strides sdc,
+                       void* control, uint64_t control_size,
                        void* workspace, uint64_t workspace_bytes, uint32_t epoch,
                        void* stream);
 

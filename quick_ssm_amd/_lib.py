@@ -22,8 +22,8 @@ EXPORTED_SYMBOLS = (
     "qssm_version",
     "qssm_error_string",
     "qssm_plan_scan",
-    "qssm_workspace_reset",
-    "qssm_workspace_status",
+    "qssm_zero_fill",
+    "qssm_control_status",
     "qssm_scan_forward",
     "qssm_scan_backward",
     "qssm_copy_bytes",
@@ -54,6 +54,7 @@ class Plan(ctypes.Structure):
         ("n_ckpt", ctypes.c_int32),
         ("lds_bytes", ctypes.c_int32),
         ("reserved", ctypes.c_int32),
+        ("control_bytes", ctypes.c_uint64),
         ("workspace_bytes", ctypes.c_uint64),
         ("ckpt_elems", ctypes.c_uint64),
     ]
@@ -86,17 +87,17 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.qssm_error_string.argtypes = []
     lib.qssm_plan_scan.restype = ctypes.c_int
     lib.qssm_plan_scan.argtypes = [i32] * 9 + [ctypes.POINTER(Plan)]
-    lib.qssm_workspace_reset.restype = ctypes.c_int
-    lib.qssm_workspace_reset.argtypes = [vp, u64, vp]
-    lib.qssm_workspace_status.restype = ctypes.c_int
-    lib.qssm_workspace_status.argtypes = [vp, vp, ctypes.POINTER(i32)]
+    lib.qssm_zero_fill.restype = ctypes.c_int
+    lib.qssm_zero_fill.argtypes = [vp, u64, vp]
+    lib.qssm_control_status.restype = ctypes.c_int
+    lib.qssm_control_status.argtypes = [vp, vp, ctypes.POINTER(i32)]
     lib.qssm_scan_forward.restype = ctypes.c_int
     lib.qssm_scan_forward.argtypes = (
-        [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, u64, ctypes.c_uint32, vp]
+        [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, u64, vp, u64, ctypes.c_uint32, vp]
     )
     lib.qssm_scan_backward.restype = ctypes.c_int
     lib.qssm_scan_backward.argtypes = (
-        [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, Strides] * 4 + [vp, u64, ctypes.c_uint32, vp]
+        [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, Strides] * 4 + [vp, u64, vp, u64, ctypes.c_uint32, vp]
     )
     lib.qssm_copy_bytes.restype = ctypes.c_int
     lib.qssm_copy_bytes.argtypes = [vp, vp, u64, vp]

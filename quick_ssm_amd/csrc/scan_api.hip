@@ -124,7 +124,7 @@ static bool tile_span_ok(const qssm_plan* pl, const void* p, int64_t sb, int64_t
   return span < ((int64_t)1 << 31);
 }
 
-static void fill_geometry(Geometry* g, const qssm_plan* pl, void* workspace, uint32_t epoch) {
+static void fill_geometry(Geometry* g, const qssm_plan* pl, void* control, void* workspace, uint32_t epoch) {
   g->B = pl->B;
   g->L = pl->L;
   g->D = pl->D;
@@ -139,9 +139,9 @@ static void fill_geometry(Geometry* g, const qssm_plan* pl, void* workspace, uin
   g->n_ckpt = pl->n_ckpt;
   g->epoch = epoch;
   char* ws = (char*)workspace;
-  g->status = (int*)ws;
-  g->tickets = (unsigned long long*)(ws + kStatusBytes);
-  g->maps = (unsigned long long*)(ws + ws_maps_offset((uint64_t)g->n_chains));
+  g->status = (int*)control;
+  g->tickets = (unsigned*)((char*)control + kStatusBytes);
+  g->maps = (unsigned long long*)ws;
   g->states = (unsigned long long*)(ws + ws_states_offset((uint64_t)g->n_chains, (uint64_t)g->n_seg,
                                                           (uint64_t)pl->strip_cols));
 }
@@ -185,21 +185,19 @@ int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int32_t ou
   while (vec > 1 && (align_elems % vec != 0 || (D > 0 && D % vec != 0))) vec >>= 1;
   plan->vec = vec;
 
-  // Steps per lane: 8 where the registers allow; the backward at 8 bytes per lane holds five
-  // operands plus h per step and stays at 4.
+  // Steps per lane: 8.  Fewer steps mean more, shorter tiles, and every tile pays the same fixed
+  // hand-over cost; 8 steps of five operands still fit the register file at two waves per SIMD.
   int steps = 8;
-  if (direction == QSSM_BACKWARD && vec * es >= 8) steps = 4;
   const int tune_steps = (tune >> 8) & 0xff;
   if (tune_steps == 4 || tune_steps == 8) steps = tune_steps;
 
   // Lanes per row: 512-byte row pieces (what HBM needs to stream at full rate) when D allows,
-  // never more lanes than the row has vectors.  Workgroup: as many time groups as the sequence
-  // can feed, up to 1024 lanes, because every tile boundary along time costs a hand-over.
+  // never more lanes than the row has vectors.  Workgroup: 256 lanes; small workgroups overlap
+  // each other's waits best, and clusters (below) keep the number of serial hand-overs down.
   const int cap = lanes_cap(D, vec);
   int g = 512 / (vec * es);
   if (g > cap) g = cap;
-  int threads = kMaxThreads;
-  if (vec == 1) threads = 256;
+  int threads = 256;
   const int tune_g = (tune & 0xff) - 1, tune_t = (tune >> 24) & 0xf;
   const bool fixed_g = tune_g >= 0 && tune_g <= 10, fixed_t = tune_t >= 1 && tune_t <= 3;
   if (fixed_g) g = 1 << tune_g;
@@ -267,13 +265,15 @@ int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int32_t ou
   plan->n_ckpt = (L + plan->ckpt_stride - 1) / plan->ckpt_stride;
 
   // Cluster size: each cluster boundary is one serial hand-over (about 1.3 us under load on
-  // MI355X); keep their number per chain at 32 or fewer when LDS allows.
+  // MI355X) that every chain pays in turn; keep their number per chain at 32 or fewer when LDS
+  // allows.  Inside a cluster a tile reads the maps of all earlier tiles, so clusters stay small.
   int cluster = 1;
   const int tune_r = (tune >> 28) & 0xf;
   if (tune_r >= 1) {
     cluster = 1 << (tune_r - 1);
   } else {
     while (cluster < 8 && (plan->n_seg + cluster - 1) / cluster > 32) cluster <<= 1;
+    if (cluster < 2 && plan->n_seg > 8) cluster = 2;
   }
   auto lds_for = [&](int r) -> size_t {
     return direction == QSSM_FORWARD ? fwd_lds_bytes(threads, vec, plan->strip_cols, r)
@@ -287,17 +287,18 @@ int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int32_t ou
 
   const uint64_t n_chains = (uint64_t)B * plan->n_strips;
   if (n_chains * plan->n_seg > 0x7fffffffull) return fail(QSSM_EINVAL, "shape needs more than 2^31 tiles");
+  plan->control_bytes = control_bytes(n_chains);
   plan->workspace_bytes = plan->n_seg > 1 ? ws_total_bytes(n_chains, (uint64_t)plan->n_seg, (uint64_t)plan->n_super,
                                                            (uint64_t)plan->strip_cols)
-                                          : ws_maps_offset(n_chains);
+                                          : 0;
   plan->ckpt_elems = (uint64_t)B * plan->n_ckpt * D;
   return 0;
 }
 
-int qssm_workspace_reset(void* workspace, uint64_t bytes, void* stream) {
+int qssm_zero_fill(void* workspace, uint64_t bytes, void* stream) {
   if (workspace == nullptr || bytes == 0) return 0;
   if (((uintptr_t)workspace) % 16 != 0 || bytes % 16 != 0)
-    return fail(QSSM_EALIGN, "workspace must be 16-byte aligned and a multiple of 16 bytes");
+    return fail(QSSM_EALIGN, "buffer must be 16-byte aligned and a multiple of 16 bytes");
   const uint64_t n16 = bytes / 16;
   uint64_t blocks = (n16 + 255) / 256;
   if (blocks > 4096) blocks = 4096;
@@ -307,9 +308,9 @@ int qssm_workspace_reset(void* workspace, uint64_t bytes, void* stream) {
   return e == hipSuccess ? 0 : hip_fail(e, "fill_zero_kernel launch");
 }
 
-int qssm_workspace_status(const void* workspace, void* stream, int32_t* status) {
-  if (workspace == nullptr || status == nullptr) return fail(QSSM_EINVAL, "NULL argument");
-  hipError_t e = hipMemcpyAsync(status, workspace, sizeof(int32_t), hipMemcpyDeviceToHost, (hipStream_t)stream);
+int qssm_control_status(const void* control, void* stream, int32_t* status) {
+  if (control == nullptr || status == nullptr) return fail(QSSM_EINVAL, "NULL argument");
+  hipError_t e = hipMemcpyAsync(status, control, sizeof(int32_t), hipMemcpyDeviceToHost, (hipStream_t)stream);
   if (e != hipSuccess) return hip_fail(e, "hipMemcpyAsync(status)");
   e = hipStreamSynchronize((hipStream_t)stream);
   return e == hipSuccess ? 0 : hip_fail(e, "hipStreamSynchronize");
@@ -317,8 +318,8 @@ int qssm_workspace_status(const void* workspace, void* stream, int32_t* status) 
 
 int qssm_scan_forward(const qssm_plan* plan, const void* x, qssm_strides sx, const void* a, qssm_strides sa,
                       const void* b, qssm_strides sb, const void* c, qssm_strides sc, void* y, qssm_strides sy,
-                      float* h_out, qssm_strides sh, float* ckpt, void* workspace, uint64_t workspace_bytes,
-                      uint32_t epoch, void* stream) {
+                      float* h_out, qssm_strides sh, float* ckpt, void* control, uint64_t control_size,
+                      void* workspace, uint64_t workspace_bytes, uint32_t epoch, void* stream) {
   int rc = check_plan(plan, QSSM_FORWARD);
   if (rc != 0) return rc;
   if (plan->B == 0 || plan->L == 0 || plan->D == 0) return 0;
@@ -331,9 +332,14 @@ int qssm_scan_forward(const qssm_plan* plan, const void* x, qssm_strides sx, con
       !aligned_to(c, sc.b, sc.l, es, v) || !aligned_to(y, sy.b, sy.l, os, v) ||
       !aligned_to(h_out, sh.b, sh.l, 4, v) || !aligned_to(ckpt, 0, 0, 4, v))
     return fail(QSSM_EALIGN, "a pointer or stride is not aligned to plan.vec=%d elements", v);
-  if (workspace == nullptr || workspace_bytes < plan->workspace_bytes)
+  if (control == nullptr || control_size < plan->control_bytes)
+    return fail(QSSM_EWORKSPACE, "control block has %llu bytes, plan needs %llu", (unsigned long long)control_size,
+                (unsigned long long)plan->control_bytes);
+  if (plan->workspace_bytes > 0 && (workspace == nullptr || workspace_bytes < plan->workspace_bytes))
     return fail(QSSM_EWORKSPACE, "workspace has %llu bytes, plan needs %llu", (unsigned long long)workspace_bytes,
                 (unsigned long long)plan->workspace_bytes);
+  if (((uintptr_t)control) % 8 != 0 || ((uintptr_t)workspace) % 8 != 0)
+    return fail(QSSM_EALIGN, "control block and workspace must be 8-byte aligned");
 
   if (epoch == 0) return fail(QSSM_EINVAL, "epoch must be nonzero");
   if (!tile_span_ok(plan, x, sx.b, sx.l, es) || !tile_span_ok(plan, a, sa.b, sa.l, es) ||
@@ -342,7 +348,7 @@ int qssm_scan_forward(const qssm_plan* plan, const void* x, qssm_strides sx, con
     return fail(QSSM_EINVAL, "a time stride is negative or too large for 32-bit tile offsets; pass a contiguous copy");
 
   FwdArgs args;
-  fill_geometry(&args.g, plan, workspace, epoch);
+  fill_geometry(&args.g, plan, control, workspace, epoch);
   args.x = x; args.a = a; args.b = b; args.c = c; args.y = y; args.h_out = h_out; args.ckpt = ckpt;
   args.x_sb = sx.b; args.x_sl = sx.l; args.a_sb = sa.b; args.a_sl = sa.l;
   args.b_sb = sb.b; args.b_sl = sb.l; args.c_sb = sc.b; args.c_sl = sc.l;
@@ -358,8 +364,8 @@ int qssm_scan_backward(const qssm_plan* plan, const void* x, qssm_strides sx, co
                        const void* b, qssm_strides sb, const void* c, qssm_strides sc, const void* dy,
                        qssm_strides sdy, const float* h, qssm_strides sh, const float* ckpt, void* dx,
                        qssm_strides sdx, void* da, qssm_strides sda, void* db, qssm_strides sdb, void* dc,
-                       qssm_strides sdc, void* workspace, uint64_t workspace_bytes, uint32_t epoch,
-                       void* stream) {
+                       qssm_strides sdc, void* control, uint64_t control_size, void* workspace,
+                       uint64_t workspace_bytes, uint32_t epoch, void* stream) {
   int rc = check_plan(plan, QSSM_BACKWARD);
   if (rc != 0) return rc;
   if (plan->B == 0 || plan->L == 0 || plan->D == 0) return 0;
@@ -375,9 +381,14 @@ int qssm_scan_backward(const qssm_plan* plan, const void* x, qssm_strides sx, co
       !aligned_to(da, sda.b, sda.l, es, v) || !aligned_to(db, sdb.b, sdb.l, es, v) ||
       !aligned_to(dc, sdc.b, sdc.l, es, v))
     return fail(QSSM_EALIGN, "a pointer or stride is not aligned to plan.vec=%d elements", v);
-  if (workspace == nullptr || workspace_bytes < plan->workspace_bytes)
+  if (control == nullptr || control_size < plan->control_bytes)
+    return fail(QSSM_EWORKSPACE, "control block has %llu bytes, plan needs %llu", (unsigned long long)control_size,
+                (unsigned long long)plan->control_bytes);
+  if (plan->workspace_bytes > 0 && (workspace == nullptr || workspace_bytes < plan->workspace_bytes))
     return fail(QSSM_EWORKSPACE, "workspace has %llu bytes, plan needs %llu", (unsigned long long)workspace_bytes,
                 (unsigned long long)plan->workspace_bytes);
+  if (((uintptr_t)control) % 8 != 0 || ((uintptr_t)workspace) % 8 != 0)
+    return fail(QSSM_EALIGN, "control block and workspace must be 8-byte aligned");
 
   if (epoch == 0) return fail(QSSM_EINVAL, "epoch must be nonzero");
   if (!tile_span_ok(plan, x, sx.b, sx.l, es) || !tile_span_ok(plan, a, sa.b, sa.l, es) ||
@@ -388,7 +399,7 @@ int qssm_scan_backward(const qssm_plan* plan, const void* x, qssm_strides sx, co
     return fail(QSSM_EINVAL, "a time stride is negative or too large for 32-bit tile offsets; pass a contiguous copy");
 
   BwdArgs args;
-  fill_geometry(&args.g, plan, workspace, epoch);
+  fill_geometry(&args.g, plan, control, workspace, epoch);
   args.x = x; args.a = a; args.b = b; args.c = c; args.dy = dy; args.h = h; args.ckpt = ckpt;
   args.dx = dx; args.da = da; args.db = db; args.dc = dc;
   args.x_sb = sx.b; args.x_sl = sx.l; args.a_sb = sa.b; args.a_sl = sa.l;

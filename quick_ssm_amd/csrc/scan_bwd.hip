@@ -42,10 +42,14 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   // ---- claim a tile of this chain, last tile in time first -----------------------------------
   int seg = 0;
   if (g.n_seg > 1) {
-    if (tid == 0) *sSeg = (int)claim_ticket(g.tickets, chain, g.epoch);
+#ifdef QSSM_PROBE_STATIC
+    const int tk = blockIdx.x / g.n_chains;
+#else
+    if (tid == 0) *sSeg = (int)claim_ticket(g.tickets, chain, g.n_seg);
     __syncthreads();
     const int tk = __builtin_amdgcn_readfirstlane(*sSeg);
-    if ((unsigned)tk >= (unsigned)g.n_seg) {  // more claims than tiles: the epoch was reused
+#endif
+    if ((unsigned)tk >= (unsigned)g.n_seg) {  // the control block was not zero on entry
       if (tid == 0) raise_status(g.status, 2);
       return;
     }
@@ -74,6 +78,29 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   const uint32_t co = (uint32_t)((j * T * (int)p.c_sl + dl) * (int)sizeof(Tin)), cs = (uint32_t)p.c_sl * sizeof(Tin);
   const uint32_t go = (uint32_t)((j * T * (int)p.dy_sl + dl) * (int)sizeof(Tout)), gs = (uint32_t)p.dy_sl * sizeof(Tout);
   const float* hp = p.h + (int64_t)bi * p.h_sb + (int64_t)t0 * p.h_sl + d;
+
+  // ---- ask for the neighbours' words first: they are looked at once the answers are back ------
+#ifdef QSSM_PROBE_NOCHAIN
+  const bool multi = false;
+#else
+  const bool multi = g.n_seg > 1;
+#endif
+  const int s = seg / R;                                     // cluster of this tile
+  const int m = seg - s * R;                                 // tiles of the cluster before this one
+  const int last = ((s + 1) * R < g.n_seg ? (s + 1) * R : g.n_seg) - 1;
+  const int cnt = last - seg;                                // tiles of the cluster after this one
+  const bool edge = (j == 0);  // the first lane group holds the tile's total reverse map
+  const int lane = tid & (G - 1);  // position inside the lane group = position inside a word plane
+  const unsigned long long* my_map = g.maps + ((int64_t)chain * g.n_seg + (seg + 1 + j)) * cols * 2 + lane;
+  const unsigned long long* next_state = g.states + ((int64_t)chain * g.n_super + (s + 1)) * cols + lane;
+  const bool want_map = multi && dok && j < cnt;                       // this lane group fetches the map of tile (seg + 1 + j)
+  const bool want_state = multi && dok && edge && s + 1 < g.n_super;   // and the first group the next cluster's carry
+  Peek<2 * VEC> pk_map;
+  Peek<VEC> pk_state;
+  pk_map.clear();
+  pk_state.clear();
+  if (want_map) pk_map.issue(my_map, G);
+  if (want_state) pk_state.issue(next_state, G);
 
   // ---- issue every load of the tile before touching any of them ------------------------------
   Words<Tin, VEC> rx[T], ra[T], rb[T], rc[T];
@@ -140,6 +167,31 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
     for (int v = 0; v < VEC; ++v) hprev[v] = hv.v[v];
   }
 
+  // ---- the neighbours' answers (they were asked for before the operands, so they are back first)
+  pk_map.pin();
+  pk_state.pin();
+  bool map_here = false, state_here = false;
+  float ein[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) ein[v] = 0.0f;
+  if (want_map && pk_map.ready(g.epoch)) {
+    map_here = true;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      sPA[j * cols + dl + v] = pk_map.value(2 * v);
+      sPX[j * cols + dl + v] = pk_map.value(2 * v + 1);
+    }
+  }
+  if (want_state && pk_state.ready(g.epoch)) {
+    state_here = true;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) ein[v] = pk_state.value(v);
+  }
+  // Second look for what was not there yet; the answers travel while sweep 1 runs.
+  const bool ask_map = want_map && !map_here, ask_state = want_state && !state_here;
+  if (ask_map) pk_map.issue(my_map, G);
+  if (ask_state) pk_state.issue(next_state, G);
+
   // ---- sweep 1: fold this lane's T steps into the forward and the reverse affine map ----------
   float A[VEC], Xf[VEC], Xe[VEC];
 #pragma unroll
@@ -169,13 +221,14 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   }
 #pragma unroll
   for (int i = 0; i < T; ++i) { forget(ra[i]); forget(rb[i]); forget(rx[i]); forget(rc[i]); forget(rg[i]); }
-  __syncthreads();
+  lds_barrier();
 
   // ---- compose: groups before this one (forward state), groups after it (reverse carry) --------
   float Ap[VEC], Xp[VEC], As[VEC], Xs[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; ++v) { Ap[v] = 1.0f; Xp[v] = 0.0f; As[v] = 1.0f; Xs[v] = 0.0f; }
   if (!have_h) {
+#pragma unroll 4
     for (int k = 0; k < j; ++k) {
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
@@ -185,6 +238,7 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
       }
     }
   }
+#pragma unroll 4
   for (int k = NG - 1; k > j; --k) {
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
@@ -195,64 +249,72 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   }
 
   // ---- reverse carry entering the tile -----------------------------------------------------------
-  float ein[VEC];
-#pragma unroll
-  for (int v = 0; v < VEC; ++v) ein[v] = 0.0f;
-  if (g.n_seg > 1) {
-    const int s = seg / R;                                     // cluster of this tile
-    const int m = seg - s * R;                                 // tiles of the cluster before this one
-    const int last = ((s + 1) * R < g.n_seg ? (s + 1) * R : g.n_seg) - 1;
-    const int cnt = last - seg;                                // tiles of the cluster after this one
-    const bool edge = (j == 0);  // the first lane group holds the tile's total reverse map
+  if (multi) {
     float At[VEC], Xt[VEC];
     if (edge) {
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) { At[v] = A[v] * As[v]; Xt[v] = A[v] * Xs[v] + Xe[v]; }
+      for (int v = 0; v < VEC; ++v) {
+        const float av = sA[tid * VEC + v];
+        At[v] = av * As[v];
+        Xt[v] = av * Xs[v] + sXe[tid * VEC + v];
+      }
       // Earlier tiles of the cluster need this tile's map; it depends on nothing, so it goes out first.
       if (dok && m > 0) {
-        unsigned long long* mw = g.maps + (((int64_t)chain * g.n_seg + seg) * cols + dl) * 2;
+        unsigned long long* mw = g.maps + ((int64_t)chain * g.n_seg + seg) * cols * 2 + lane;
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
-          word_publish(mw + 2 * v, g.epoch, At[v]);
-          word_publish(mw + 2 * v + 1, g.epoch, Xt[v]);
+          word_publish(mw + (2 * v) * G, g.epoch, At[v]);
+          word_publish(mw + (2 * v + 1) * G, g.epoch, Xt[v]);
         }
       }
     }
-    if (cnt > 0) {
-      // Lane group j fetches the maps of the later tiles seg+1+j, seg+1+j+NG, ... of the cluster.
-      for (int i = j; i < cnt; i += NG) {
-        if (dok) {
-          float w[2 * VEC];
-          const unsigned long long* mw = g.maps + (((int64_t)chain * g.n_seg + (seg + 1 + i)) * cols + dl) * 2;
-          if (!words_wait<2 * VEC>(mw, g.epoch, w)) raise_status(g.status, 1);
+    // The second look's answers.
+    if (ask_map && pk_map.ready(g.epoch)) {
+      map_here = true;
 #pragma unroll
-          for (int v = 0; v < VEC; ++v) {
-            sPA[i * cols + dl + v] = w[2 * v];
-            sPX[i * cols + dl + v] = w[2 * v + 1];
-          }
+      for (int v = 0; v < VEC; ++v) {
+        sPA[j * cols + dl + v] = pk_map.value(2 * v);
+        sPX[j * cols + dl + v] = pk_map.value(2 * v + 1);
+      }
+    }
+    if (ask_state && pk_state.ready(g.epoch)) {
+      state_here = true;
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) ein[v] = pk_state.value(v);
+    }
+    // Whatever is still missing is waited for: lane group j takes the maps of the later tiles
+    // seg+1+j, seg+1+j+NG, ... of the cluster, and the first group, at the same time, the carry the
+    // next cluster in time hands back (the one serial hop of the launch).
+    for (int i = j; i < cnt; i += NG) {
+      if (dok && !(i == j && map_here)) {
+        float w[2 * VEC];
+        const unsigned long long* mw = g.maps + ((int64_t)chain * g.n_seg + (seg + 1 + i)) * cols * 2 + lane;
+        if (!words_wait<2 * VEC, false>(mw, G, g.epoch, w)) raise_status(g.status, 1);
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          sPA[i * cols + dl + v] = w[2 * v];
+          sPX[i * cols + dl + v] = w[2 * v + 1];
         }
       }
-      __syncthreads();
     }
+    if (want_state && !state_here) {
+      if (!words_wait<VEC, true>(next_state, G, g.epoch, ein)) raise_status(g.status, 1);
+    }
+    if (cnt > 0) lds_barrier();
     if (edge) {
-      // The one serial hop: the carry the next cluster in time hands back.
-      if (dok && s + 1 < g.n_super) {
-        const unsigned long long* sw = g.states + ((int64_t)chain * g.n_super + (s + 1)) * cols + dl;
-        if (!words_wait<VEC>(sw, g.epoch, ein)) raise_status(g.status, 1);
-      }
       for (int i = cnt - 1; i >= 0; --i) {
 #pragma unroll
         for (int v = 0; v < VEC; ++v) ein[v] = sPA[i * cols + dl + v] * ein[v] + sPX[i * cols + dl + v];
       }
       if (dok && m == 0 && s > 0) {
-        unsigned long long* sw = g.states + ((int64_t)chain * g.n_super + s) * cols + dl;
+        unsigned long long* sw = g.states + ((int64_t)chain * g.n_super + s) * cols + lane;
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) word_publish(sw + v, g.epoch, At[v] * ein[v] + Xt[v]);
+        for (int v = 0; v < VEC; ++v) word_publish(sw + v * G, g.epoch, At[v] * ein[v] + Xt[v]);
       }
 #pragma unroll
       for (int v = 0; v < VEC; ++v) sE[dl + v] = ein[v];
     }
-    __syncthreads();
+    lds_barrier();
 #pragma unroll
     for (int v = 0; v < VEC; ++v) ein[v] = sE[dl + v];
   }

@@ -21,9 +21,15 @@
 // Words exchanged between workgroups are {epoch:32 | fp32 bits:32}: flag and payload travel
 // in one 64-bit access, so no fence is needed between them, and a word left over from an
 // earlier launch (older epoch) reads as "not there yet".  Agent scope makes the accesses
-// coherent across the XCDs' separate L2 caches.  Tiles of a chain are claimed in time order
-// through a per-chain ticket counter (also epoch-tagged), so every tile a workgroup waits for
-// was claimed by a workgroup that is already running.
+// coherent across the XCDs' separate L2 caches.  A tile asks for its neighbours' words before
+// it issues its own operand loads and looks at the answers when they are back; in steady
+// state (tiles are claimed in time order, so neighbours ran a generation earlier) the words
+// are there and the hand-over costs no extra round trip.
+//
+// Tiles of a chain are claimed in time order through a per-chain ticket counter in a small
+// control block, so every tile a workgroup waits for was claimed by a workgroup that is already
+// running.  The control block holds nothing but the status word and the counters; the holder of
+// a chain's last ticket puts its counter back to zero.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -33,22 +39,23 @@
 
 namespace qssm {
 
-// Polls before a tile gives up on a neighbour's word (each poll is a round trip to the
-// coherent level of the memory system plus a short sleep: roughly a second in total).
+// Polls before a tile gives up on a neighbour's word.  Each poll is a round trip to the
+// coherent level of the memory system plus a sleep of up to half a microsecond: about a second
+// in total.
 constexpr int kSpinLimit = 1 << 20;
 
-// Workspace layout (bytes): [0,64) status word; one 64-byte slot per chain holding its ticket
-// counter; then, 256-byte aligned, the tile maps (2 words per column per tile); then the
-// cluster states (1 word per column per cluster).
+// Control block layout (bytes): [0,64) status word; then one 64-byte slot per chain holding its
+// ticket counter.  Workspace layout: the tile maps (2 words per column per tile), then,
+// 256-byte aligned, the cluster states (1 word per column per cluster).
 constexpr uint64_t kStatusBytes = 64;
 constexpr uint64_t kTicketStride = 64;
 
 __host__ __device__ inline uint64_t ws_align(uint64_t off) { return (off + 255u) & ~uint64_t(255); }
-__host__ __device__ inline uint64_t ws_maps_offset(uint64_t n_chains) {
+__host__ __device__ inline uint64_t control_bytes(uint64_t n_chains) {
   return ws_align(kStatusBytes + n_chains * kTicketStride);
 }
 __host__ __device__ inline uint64_t ws_states_offset(uint64_t n_chains, uint64_t n_seg, uint64_t cols) {
-  return ws_align(ws_maps_offset(n_chains) + n_chains * n_seg * cols * 16u);
+  return ws_align(n_chains * n_seg * cols * 16u);
 }
 __host__ __device__ inline uint64_t ws_total_bytes(uint64_t n_chains, uint64_t n_seg, uint64_t n_super,
                                                    uint64_t cols) {
@@ -198,6 +205,15 @@ __device__ __forceinline__ void forget(Words<T, V>& p) {
   for (int k = 0; k < Words<T, V>::N; ++k) asm volatile("" : "+v"(p.w[k]));
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
+// outstanding global load and store of the wave (operands still in flight, words just published
+// to other workgroups), which would put a memory round trip into each of the tile's barriers.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // ---- words exchanged between workgroups ------------------------------------------------------
 
 __device__ __forceinline__ void word_publish(unsigned long long* w, unsigned epoch, float v) {
@@ -205,44 +221,87 @@ __device__ __forceinline__ void word_publish(unsigned long long* w, unsigned epo
   __hip_atomic_store(w, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Wait until N consecutive words carry this launch's epoch; all N loads of a round are in
-// flight together.  Returns false (and NaN payloads) if they never all arrive.
+// One look at N consecutive words (all N loads in flight together).
 template <int N>
-__device__ __forceinline__ bool words_wait(const unsigned long long* w, unsigned epoch, float* out) {
-  for (int spins = 0; spins < kSpinLimit; ++spins) {
-    unsigned long long r[N];
+struct Peek {
+  unsigned long long r[N];
+  // Start from "nothing there" (epoch 0 is never used), so that lanes which do not ask keep
+  // defined values and no branch has to be joined, and waited for, before later loads go out.
+  __device__ __forceinline__ void clear() {
+#pragma unroll
+    for (int n = 0; n < N; ++n) r[n] = 0ull;
+  }
+  // Word n of this lane sits at w + n * plane: the lanes of a group are adjacent within a plane,
+  // so that one load (or store) instruction of a wavefront covers whole cache lines.  Publishing
+  // 8-byte words scattered one per 32 or 64 bytes would reach memory as partial-line writes.
+  __device__ __forceinline__ void issue(const unsigned long long* w, int plane) {
 #pragma unroll
     for (int n = 0; n < N; ++n)
-      r[n] = __hip_atomic_load(const_cast<unsigned long long*>(w) + n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      r[n] = __hip_atomic_load(const_cast<unsigned long long*>(w) + (size_t)n * plane, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+  }
+  // Compiler fence: whatever looks at the answers stays behind the memory operations issued
+  // before this point (the operand loads), instead of being hoisted in front of them.
+  __device__ __forceinline__ void pin() {
+#pragma unroll
+    for (int n = 0; n < N; ++n) asm volatile("" : "+v"(r[n]) : : "memory");
+  }
+  __device__ __forceinline__ bool ready(unsigned epoch) const {
     bool ok = true;
 #pragma unroll
     for (int n = 0; n < N; ++n) ok = ok && ((unsigned)(r[n] >> 32) == epoch);
-    if (ok) {
+    return ok;
+  }
+  __device__ __forceinline__ float value(int n) const { return __uint_as_float((unsigned)r[n]); }
+};
+
+// Wait until this lane's N words (at w + n * plane) carry this launch's epoch.  While waiting, a
+// wavefront polls ONE word (its first active lane's first word, read by every lane at the same
+// address, i.e. one 8-byte request); only when that one has arrived do the lanes read their own
+// words, which the producer stored with the same instructions and which are then there as a rule.
+// This keeps a waiting tile's traffic at a few bytes per poll instead of a full row of words.
+// Returns false (and NaN payloads) if the words never arrive.
+template <int N, bool URGENT>
+__device__ __forceinline__ bool words_wait(const unsigned long long* w, int plane, unsigned epoch, float* out) {
+  const uint64_t mine = reinterpret_cast<uint64_t>(w);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)mine);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(mine >> 32));
+  unsigned long long* lead = reinterpret_cast<unsigned long long*>(((uint64_t)hi << 32) | lo);
+  // URGENT: the hand-over between clusters is the one serial path of the whole launch, so that
+  // waiter polls almost back to back at first and backs off (to about half a microsecond between
+  // polls) only when the wait drags on.  Everything else is needed later than it is published as
+  // a rule, and is polled at the slow rate from the start, so that waiting tiles do not load the
+  // memory system.
+  for (int spins = 0; spins < kSpinLimit; ++spins) {
+    const unsigned long long first = __hip_atomic_load(lead, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((unsigned)(first >> 32) == epoch) {
+      Peek<N> pk;
+      pk.issue(w, plane);
+      if (pk.ready(epoch)) {
 #pragma unroll
-      for (int n = 0; n < N; ++n) out[n] = __uint_as_float((unsigned)r[n]);
-      return true;
+        for (int n = 0; n < N; ++n) out[n] = pk.value(n);
+        return true;
+      }
     }
-    __builtin_amdgcn_s_sleep(1);
+    if (URGENT && spins < 32) {
+      __builtin_amdgcn_s_sleep(1);
+    } else {
+      const int nap = (URGENT && spins < 256) ? 2 : 8;
+      for (int k = 0; k < nap; ++k) __builtin_amdgcn_s_sleep(2);
+    }
   }
 #pragma unroll
   for (int n = 0; n < N; ++n) out[n] = __uint_as_float(0x7fc00000u);
   return false;
 }
 
-// Claim the next tile of `chain` in time order.  A ticket slot is {epoch:32 | count:32} like
-// every other word of the workspace: a slot that still carries another launch's epoch (or
-// anything else an earlier launch with a different layout left there) counts as zero, so the
-// workspace never has to be put back in order between launches.
-__device__ __forceinline__ unsigned claim_ticket(unsigned long long* tickets, int chain, unsigned epoch) {
-  unsigned long long* slot = tickets + (size_t)chain * (kTicketStride / sizeof(unsigned long long));
-  unsigned long long old = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  for (;;) {
-    const bool mine = (unsigned)(old >> 32) == epoch;
-    const unsigned long long next = mine ? old + 1ull : (((unsigned long long)epoch << 32) | 1ull);
-    if (__hip_atomic_compare_exchange_strong(slot, &old, next, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
-                                             __HIP_MEMORY_SCOPE_AGENT))
-      return mine ? (unsigned)old : 0u;
-  }
+// Claim the next tile of `chain` in time order: one atomic add.  The holder of the last ticket
+// puts the counter back to zero; by then every other tile of the chain has taken its ticket.
+__device__ __forceinline__ unsigned claim_ticket(unsigned* tickets, int chain, int n_seg) {
+  unsigned* slot = tickets + (size_t)chain * (kTicketStride / sizeof(unsigned));
+  const unsigned tk = __hip_atomic_fetch_add(slot, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (tk == (unsigned)(n_seg - 1)) __hip_atomic_store(slot, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return tk;
 }
 
 __device__ __forceinline__ void raise_status(int* status, int code) {
@@ -264,9 +323,9 @@ struct Geometry {
   int n_ckpt;       // saved states per (batch, column)
   unsigned epoch;   // this launch's flag value (nonzero)
   int* status;
-  unsigned long long* tickets;
-  unsigned long long* maps;    // [chain][tile][col][2]: the tile's affine map (A, X)
-  unsigned long long* states;  // [chain][cluster][col]: state handed to the next cluster
+  unsigned* tickets;
+  unsigned long long* maps;    // [chain][tile][2 * VEC planes][G lanes]: the tile's affine map (A, X)
+  unsigned long long* states;  // [chain][cluster][VEC planes][G lanes]: state handed to the next cluster
 };
 
 struct FwdArgs {

@@ -31,15 +31,26 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   // ---- claim a tile of this chain, in time order -------------------------------------------
   int seg = 0;
   if (g.n_seg > 1) {
-    if (tid == 0) *sSeg = (int)claim_ticket(g.tickets, chain, g.epoch);
+#ifdef QSSM_PROBE_STATIC
+    seg = blockIdx.x / g.n_chains;
+#else
+    if (tid == 0) *sSeg = (int)claim_ticket(g.tickets, chain, g.n_seg);
     __syncthreads();
     seg = __builtin_amdgcn_readfirstlane(*sSeg);
-    if ((unsigned)seg >= (unsigned)g.n_seg) {  // more claims than tiles: the epoch was reused
+#endif
+    if ((unsigned)seg >= (unsigned)g.n_seg) {  // the control block was not zero on entry
       if (tid == 0) raise_status(g.status, 2);
       return;
     }
   }
 
+#ifdef QSSM_PROBE_TIMELINE
+  unsigned long long* stamps = g.states + (int64_t)g.n_chains * g.n_super * (G * VEC) + ((int64_t)chain * g.n_seg + seg) * 8;
+#define QSSM_STAMP(k) do { if (tid == NTH - 1) stamps[k] = wall_clock64(); } while (0)
+  QSSM_STAMP(0);
+#else
+#define QSSM_STAMP(k) do {} while (0)
+#endif
   const int bi = chain / g.n_strips;
   const int strip = chain - bi * g.n_strips;
   const int j = tid >> g.g_log2;         // lane group = time sub-segment
@@ -61,6 +72,27 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   const uint32_t co = (uint32_t)((j * T * (int)p.c_sl + dl) * (int)sizeof(Tin)), cs = (uint32_t)p.c_sl * sizeof(Tin);
   const bool want_y = p.y != nullptr;
   const bool has_c = want_y && p.c != nullptr;
+
+  // ---- ask for the neighbours' words first: they are looked at once the answers are back ------
+#ifdef QSSM_PROBE_NOCHAIN
+  const bool multi = false;
+#else
+  const bool multi = g.n_seg > 1;
+#endif
+  const int s = seg / R;               // cluster of this tile
+  const int m = seg - s * R;           // tiles of the cluster before this one
+  const bool edge = (j == NG - 1);     // the last lane group holds the tile's total map
+  const int lane = tid & (G - 1);      // position inside the lane group = position inside a word plane
+  const unsigned long long* my_map = g.maps + ((int64_t)chain * g.n_seg + (seg - m + j)) * cols * 2 + lane;
+  const unsigned long long* prev_state = g.states + ((int64_t)chain * g.n_super + (s - 1)) * cols + lane;
+  const bool want_map = multi && dok && j < m;            // this lane group fetches the map of tile (seg - m + j)
+  const bool want_state = multi && dok && edge && s > 0;  // and the last group the previous cluster's state
+  Peek<2 * VEC> pk_map;
+  Peek<VEC> pk_state;
+  pk_map.clear();
+  pk_state.clear();
+  if (want_map) pk_map.issue(my_map, G);
+  if (want_state) pk_state.issue(prev_state, G);
 
   // ---- issue every load of the tile before touching any of them ------------------------------
   Words<Tin, VEC> rx[T], ra[T], rb[T], rc[T];
@@ -96,6 +128,31 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
     }
   }
 
+  // ---- the neighbours' answers (they were asked for before the operands, so they are back first)
+  pk_map.pin();
+  pk_state.pin();
+  bool map_here = false, state_here = false;
+  float hin[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) hin[v] = 0.0f;
+  if (want_map && pk_map.ready(g.epoch)) {
+    map_here = true;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      sPA[j * cols + dl + v] = pk_map.value(2 * v);
+      sPX[j * cols + dl + v] = pk_map.value(2 * v + 1);
+    }
+  }
+  if (want_state && pk_state.ready(g.epoch)) {
+    state_here = true;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) hin[v] = pk_state.value(v);
+  }
+  // Second look for what was not there yet; the answers travel while sweep 1 runs.
+  const bool ask_map = want_map && !map_here, ask_state = want_state && !state_here;
+  if (ask_map) pk_map.issue(my_map, G);
+  if (ask_state) pk_state.issue(prev_state, G);
+
   // ---- sweep 1: fold this lane's T steps into one affine map ---------------------------------
   float A[VEC], X[VEC];
 #pragma unroll
@@ -117,12 +174,15 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   }
 #pragma unroll
   for (int i = 0; i < T; ++i) { forget(ra[i]); forget(rb[i]); forget(rx[i]); }
-  __syncthreads();
+  QSSM_STAMP(1);
+  lds_barrier();
+  QSSM_STAMP(2);
 
   // ---- compose the maps of the lane groups before this one ------------------------------------
   float Ap[VEC], Xp[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; ++v) { Ap[v] = 1.0f; Xp[v] = 0.0f; }
+#pragma unroll 4
   for (int k = 0; k < j; ++k) {
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
@@ -133,65 +193,79 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   }
 
   // ---- state entering the tile ------------------------------------------------------------------
-  float hin[VEC];
-#pragma unroll
-  for (int v = 0; v < VEC; ++v) hin[v] = 0.0f;
-  if (g.n_seg > 1) {
-    const int s = seg / R;       // cluster of this tile
-    const int m = seg - s * R;   // tiles of the cluster before this one
-    const bool edge = (j == NG - 1);  // the last lane group holds the tile's total map
+  if (multi) {
     float At[VEC], Xt[VEC];
     if (edge) {
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) { At[v] = A[v] * Ap[v]; Xt[v] = A[v] * Xp[v] + X[v]; }
+      for (int v = 0; v < VEC; ++v) {
+        const float av = sA[tid * VEC + v];
+        At[v] = av * Ap[v];
+        Xt[v] = av * Xp[v] + sX[tid * VEC + v];
+      }
       // Later tiles of the cluster need this tile's map; it depends on nothing, so it goes out first.
       if (dok && m + 1 < R && seg + 1 < g.n_seg) {
-        unsigned long long* mw = g.maps + (((int64_t)chain * g.n_seg + seg) * cols + dl) * 2;
+        unsigned long long* mw = g.maps + ((int64_t)chain * g.n_seg + seg) * cols * 2 + lane;
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
-          word_publish(mw + 2 * v, g.epoch, At[v]);
-          word_publish(mw + 2 * v + 1, g.epoch, Xt[v]);
+          word_publish(mw + (2 * v) * G, g.epoch, At[v]);
+          word_publish(mw + (2 * v + 1) * G, g.epoch, Xt[v]);
         }
       }
     }
-    if (m > 0) {
-      // Lane group j fetches the maps of the earlier tiles j, j+NG, ... of the cluster.
-      for (int i = j; i < m; i += NG) {
-        if (dok) {
-          float w[2 * VEC];
-          const unsigned long long* mw = g.maps + (((int64_t)chain * g.n_seg + (seg - m + i)) * cols + dl) * 2;
-          if (!words_wait<2 * VEC>(mw, g.epoch, w)) raise_status(g.status, 1);
+    // The second look's answers.
+    if (ask_map && pk_map.ready(g.epoch)) {
+      map_here = true;
 #pragma unroll
-          for (int v = 0; v < VEC; ++v) {
-            sPA[i * cols + dl + v] = w[2 * v];
-            sPX[i * cols + dl + v] = w[2 * v + 1];
-          }
+      for (int v = 0; v < VEC; ++v) {
+        sPA[j * cols + dl + v] = pk_map.value(2 * v);
+        sPX[j * cols + dl + v] = pk_map.value(2 * v + 1);
+      }
+    }
+    if (ask_state && pk_state.ready(g.epoch)) {
+      state_here = true;
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) hin[v] = pk_state.value(v);
+    }
+    // Whatever is still missing is waited for: lane group j takes the maps of the earlier tiles
+    // j, j+NG, ... of the cluster, and the last group, at the same time, the previous cluster's
+    // state (the one serial hop of the launch).
+    for (int i = j; i < m; i += NG) {
+      if (dok && !(i == j && map_here)) {
+        float w[2 * VEC];
+        const unsigned long long* mw = g.maps + ((int64_t)chain * g.n_seg + (seg - m + i)) * cols * 2 + lane;
+        if (!words_wait<2 * VEC, false>(mw, G, g.epoch, w)) raise_status(g.status, 1);
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          sPA[i * cols + dl + v] = w[2 * v];
+          sPX[i * cols + dl + v] = w[2 * v + 1];
         }
       }
-      __syncthreads();
     }
+    QSSM_STAMP(3);
+    if (want_state && !state_here) {
+      if (!words_wait<VEC, true>(prev_state, G, g.epoch, hin)) raise_status(g.status, 1);
+    }
+    QSSM_STAMP(4);
+    if (m > 0) lds_barrier();
+    QSSM_STAMP(5);
     if (edge) {
-      // The one serial hop: the state the previous cluster ended with.
-      if (dok && s > 0) {
-        const unsigned long long* sw = g.states + ((int64_t)chain * g.n_super + (s - 1)) * cols + dl;
-        if (!words_wait<VEC>(sw, g.epoch, hin)) raise_status(g.status, 1);
-      }
       for (int i = 0; i < m; ++i) {
 #pragma unroll
         for (int v = 0; v < VEC; ++v) hin[v] = sPA[i * cols + dl + v] * hin[v] + sPX[i * cols + dl + v];
       }
       if (dok && m == R - 1 && s + 1 < g.n_super) {
-        unsigned long long* sw = g.states + ((int64_t)chain * g.n_super + s) * cols + dl;
+        unsigned long long* sw = g.states + ((int64_t)chain * g.n_super + s) * cols + lane;
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) word_publish(sw + v, g.epoch, At[v] * hin[v] + Xt[v]);
+        for (int v = 0; v < VEC; ++v) word_publish(sw + v * G, g.epoch, At[v] * hin[v] + Xt[v]);
       }
 #pragma unroll
       for (int v = 0; v < VEC; ++v) sH[dl + v] = hin[v];
     }
-    __syncthreads();
+    lds_barrier();
 #pragma unroll
     for (int v = 0; v < VEC; ++v) hin[v] = sH[dl + v];
   }
+  QSSM_STAMP(6);
 
   float h[VEC];
 #pragma unroll
@@ -227,6 +301,7 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
     // would hold an fp32 copy of the whole tile in registers.
     __builtin_amdgcn_sched_barrier(0);
   }
+  QSSM_STAMP(7);
 }
 
 template <typename Tin, typename Tout>

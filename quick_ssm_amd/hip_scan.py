@@ -28,9 +28,21 @@ _BUILT_OUT = {
 }
 
 _ws_lock = threading.Lock()
-# (device index, stream handle) -> [workspace tensor, last epoch used on it]
-_workspaces: Dict[Tuple[int, int], list] = {}
 _EPOCH_MAX = 0xFFFFFFFF
+
+
+class _Buffers:
+    """Per (device, stream): the control block, the workspace and the epoch counter that goes with it."""
+
+    __slots__ = ("control", "workspace", "epoch")
+
+    def __init__(self):
+        self.control: Optional[Tensor] = None
+        self.workspace: Optional[Tensor] = None
+        self.epoch = 0
+
+
+_buffers: Dict[Tuple[int, int], _Buffers] = {}
 
 
 def kernel_dtypes(in_dtypes: Sequence[torch.dtype], out_dtype: torch.dtype) -> Tuple[torch.dtype, torch.dtype]:
@@ -83,44 +95,47 @@ def _align_elems(tensors: Sequence[Optional[Tensor]], D: int) -> int:
     return 1
 
 
-def _workspace(device: torch.device, stream: int, nbytes: int) -> Tuple[Tensor, int]:
-    """Workspace for (device, stream), grown on demand, and the epoch for the next launch on it.
+def _launch_buffers(device: torch.device, stream: int, plan: Plan) -> Tuple[Tensor, Tensor, int]:
+    """Control block, workspace and epoch for the next launch on (device, stream).
 
-    A workspace is zero-filled when it is allocated (torch.zeros runs a fill kernel on the current
-    stream, ahead of the launch that uses it).  Every launch then gets the next epoch value, so words
-    written by earlier launches never look valid; when the 32-bit counter is used up the buffer is
-    replaced by a fresh zeroed one.
+    Both buffers are zero-filled when they are allocated (torch.zeros runs a fill kernel on the
+    current stream, ahead of the launch that uses them) and grown on demand.  The control block is
+    left zero by every launch.  The workspace is never cleared: every launch gets the next epoch
+    value, and when the 32-bit counter is used up the workspace is replaced by a fresh zeroed one.
     """
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
     with _ws_lock:
-        entry = _workspaces.get(key)
-        if entry is None or entry[0].numel() < nbytes or entry[1] >= _EPOCH_MAX:
-            size = max(1 << 20, 1 << (int(nbytes) - 1).bit_length())
-            entry = [torch.zeros(size, dtype=torch.uint8, device=device), 0]
-            _workspaces[key] = entry
-        entry[1] += 1
-        return entry[0], entry[1]
+        buf = _buffers.get(key)
+        if buf is None:
+            buf = _buffers[key] = _Buffers()
+        need_c, need_w = int(plan.control_bytes), max(int(plan.workspace_bytes), 256)
+        if buf.control is None or buf.control.numel() < need_c:
+            buf.control = torch.zeros(max(1 << 16, 1 << (need_c - 1).bit_length()), dtype=torch.uint8, device=device)
+        if buf.workspace is None or buf.workspace.numel() < need_w or buf.epoch >= _EPOCH_MAX:
+            buf.workspace = torch.zeros(max(1 << 20, 1 << (need_w - 1).bit_length()), dtype=torch.uint8, device=device)
+            buf.epoch = 0
+        buf.epoch += 1
+        return buf.control, buf.workspace, buf.epoch
 
 
 def workspace_status(device: Optional[torch.device] = None) -> int:
-    """Status word of the current stream's workspace (synchronises).  0 = all launches completed."""
+    """Status word of the current stream's control block (synchronises).  0 = all launches completed."""
     device = torch.device("cuda", torch.cuda.current_device()) if device is None else device
     stream = torch.cuda.current_stream(device).cuda_stream
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
     with _ws_lock:
-        entry = _workspaces.get(key)
-    if entry is None:
+        buf = _buffers.get(key)
+    if buf is None or buf.control is None:
         return 0
-    ws = entry[0]
     out = ctypes.c_int32(0)
-    _lib.check(_lib.load().qssm_workspace_status(ws.data_ptr(), stream, ctypes.byref(out)))
+    _lib.check(_lib.load().qssm_control_status(buf.control.data_ptr(), stream, ctypes.byref(out)))
     return int(out.value)
 
 
 def reset_workspaces() -> None:
-    """Drop every cached workspace (the next launch allocates a fresh zeroed one)."""
+    """Drop every cached buffer (the next launch allocates fresh zeroed ones)."""
     with _ws_lock:
-        _workspaces.clear()
+        _buffers.clear()
 
 
 def make_plan(B: int, L: int, D: int, in_dtype: torch.dtype, out_dtype: torch.dtype, direction: int,
@@ -182,13 +197,13 @@ def scan_forward(
 
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
-        ws, epoch = _workspace(dev, stream, int(plan.workspace_bytes))
+        ctl, ws, epoch = _launch_buffers(dev, stream, plan)
         _lib.check(
             _lib.load().qssm_scan_forward(
                 ctypes.byref(plan),
                 _ptr(x), _strides(x), _ptr(a), _strides(a), _ptr(b), _strides(b), _ptr(c), _strides(c),
                 _ptr(y), _strides(y), _ptr(h), _strides(h), _ptr(ckpt),
-                ws.data_ptr(), ws.numel(), epoch, stream,
+                ctl.data_ptr(), ctl.numel(), ws.data_ptr(), ws.numel(), epoch, stream,
             )
         )
     return y, h, ckpt, int(plan.ckpt_stride)
@@ -228,7 +243,7 @@ def scan_backward(
 
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
-        ws, epoch = _workspace(dev, stream, int(plan.workspace_bytes))
+        ctl, ws, epoch = _launch_buffers(dev, stream, plan)
         _lib.check(
             _lib.load().qssm_scan_backward(
                 ctypes.byref(plan),
@@ -236,7 +251,7 @@ def scan_backward(
                 _ptr(dy), _strides(dy), _ptr(h), _strides(h), _ptr(ckpt),
                 _ptr(grads[0]), _strides(grads[0]), _ptr(grads[1]), _strides(grads[1]),
                 _ptr(grads[2]), _strides(grads[2]), _ptr(grads[3]), _strides(grads[3]),
-                ws.data_ptr(), ws.numel(), epoch, stream,
+                ctl.data_ptr(), ctl.numel(), ws.data_ptr(), ws.numel(), epoch, stream,
             )
         )
     return tuple(grads)

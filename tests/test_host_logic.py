@@ -19,7 +19,7 @@ def test_library_exports_every_declared_symbol(hip_lib):
     for name in declared:
         assert getattr(hip_lib, name) is not None
     assert hip_lib.qssm_version() == 100
-    assert ctypes.sizeof(_lib.Plan) == 20 * 4 + 2 * 8
+    assert ctypes.sizeof(_lib.Plan) == 20 * 4 + 3 * 8
 
 
 def test_chunk_ranges_follow_the_reference_rules():
@@ -80,9 +80,9 @@ def test_plan_rejects_bad_arguments(hip_lib):
 def test_launchers_validate_before_touching_the_gpu(hip_lib):
     plan = hip_scan.make_plan(2, 64, 8, torch.float32, torch.float32, _lib.QSSM_FORWARD, 4)
     z = _lib.Strides(0, 0)
-    args = [ctypes.byref(plan)] + [None, z] * 6 + [None, None, 0, 1, None]
+    args = [ctypes.byref(plan)] + [None, z] * 6 + [None, None, 0, None, 0, 1, None]
     assert hip_lib.qssm_scan_forward(*args) == _lib.QSSM_EINVAL      # NULL operands
-    bwd = [ctypes.byref(plan)] + [None, z] * 6 + [None] + [None, z] * 4 + [None, 0, 1, None]
+    bwd = [ctypes.byref(plan)] + [None, z] * 6 + [None] + [None, z] * 4 + [None, 0, None, 0, 1, None]
     assert hip_lib.qssm_scan_backward(*bwd) == _lib.QSSM_EINVAL      # forward plan given to the backward
     assert b"direction" in hip_lib.qssm_error_string()
     assert hip_lib.qssm_copy_bytes(8, 16, 10, None) == _lib.QSSM_EALIGN
@@ -161,8 +161,9 @@ def _tile_accesses(plan, B, L, D):
     n_chains = B * plan.n_strips
     hi_elem, hi_ckpt, hi_word = -1, -1, -1
     lo_elem = 0
-    maps_off = (64 + n_chains * 64 + 255) // 256 * 256
-    states_off = (maps_off + n_chains * plan.n_seg * cols * 16 + 255) // 256 * 256
+    maps_off = 0
+    states_off = (n_chains * plan.n_seg * cols * 16 + 255) // 256 * 256
+    assert plan.control_bytes >= 64 + n_chains * 64
     for chain in range(n_chains):
         bi, strip = divmod(chain, plan.n_strips)
         d = strip * cols + dl
