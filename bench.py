@@ -177,7 +177,7 @@ def main() -> int:
                                 args.steps, args.warmup)
         del src, dst
     status = hip_scan.workspace_status()
-    align = 4 if D % 4 == 0 else (2 if D % 2 == 0 else 1)
+    align = hip_scan._align_elems([xd, ad, bd, cd, dy], D)   # what the timed launches were planned with
     plan_b = hip_scan.make_plan(B, L, D, dtype, out_dtype, _lib.QSSM_BACKWARD, align, stride, args.tune_bwd)
     plan_f = hip_scan.make_plan(B, L, D, dtype, out_dtype, _lib.QSSM_FORWARD, align, stride, args.tune_fwd)
 

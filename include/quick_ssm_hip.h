@@ -102,7 +102,7 @@ QSSM_API const char* qssm_error_string(void);
 
 /*
  * Choose the launch geometry for a shape.
- *   align_elems : largest power of two (<= 4) that divides D, every batch/time stride, and
+ *   align_elems : largest power of two (<= 8) that divides D, every batch/time stride, and
  *                 every base address expressed in elements, over all tensors of the launch.
  *   ckpt_stride : 0 lets the forward plan pick; a backward plan (and a forward plan that must
  *                 match one) passes the stride the saved states were written with.

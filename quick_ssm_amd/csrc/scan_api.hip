@@ -198,6 +198,9 @@ int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int32_t ou
   int g = 512 / (vec * es);
   if (g > cap) g = cap;
   int threads = 256;
+  // The forward for 16-bit storage keeps c in LDS when rows can be fetched 16 bytes at a time, which
+  // leaves room for two 512-lane workgroups per compute unit: tiles twice as long, half the hand-overs.
+  if (direction == QSSM_FORWARD && es == 2 && vec == 4 && steps == 8 && align_elems % 8 == 0) threads = 512;
   const int tune_g = (tune & 0xff) - 1, tune_t = (tune >> 24) & 0xf;
   const bool fixed_g = tune_g >= 0 && tune_g <= 10, fixed_t = tune_t >= 1 && tune_t <= 3;
   if (fixed_g) g = 1 << tune_g;
@@ -264,15 +267,16 @@ int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int32_t ou
   plan->n_seg = (L + plan->seg_len - 1) / plan->seg_len;
   plan->n_ckpt = (L + plan->ckpt_stride - 1) / plan->ckpt_stride;
 
-  // Cluster size: each cluster boundary is one serial hand-over (about 1.3 us under load on
-  // MI355X) that every chain pays in turn; keep their number per chain at 32 or fewer when LDS
-  // allows.  Inside a cluster a tile reads the maps of all earlier tiles, so clusters stay small.
+  // Cluster size: each cluster boundary is one serial hand-over (about 2 us under load on MI355X)
+  // that every chain pays in turn; keep their number per chain at 64 or fewer when LDS allows.
+  // Inside a cluster a tile reads the maps of all earlier tiles, and every exchanged word lengthens
+  // the tile's stay on its compute unit, so clusters stay small.
   int cluster = 1;
   const int tune_r = (tune >> 28) & 0xf;
   if (tune_r >= 1) {
     cluster = 1 << (tune_r - 1);
   } else {
-    while (cluster < 8 && (plan->n_seg + cluster - 1) / cluster > 32) cluster <<= 1;
+    while (cluster < 8 && (plan->n_seg + cluster - 1) / cluster > 64) cluster <<= 1;
     if (cluster < 2 && plan->n_seg > 8) cluster = 2;
   }
   auto lds_for = [&](int r) -> size_t {
@@ -354,7 +358,15 @@ int qssm_scan_forward(const qssm_plan* plan, const void* x, qssm_strides sx, con
   args.b_sb = sb.b; args.b_sl = sb.l; args.c_sb = sc.b; args.c_sl = sc.l;
   args.y_sb = sy.b; args.y_sl = sy.l; args.h_sb = sh.b; args.h_sl = sh.l;
   const dim3 grid((unsigned)((uint64_t)args.g.n_chains * args.g.n_seg));
-  if (!fn(args, plan->vec, plan->steps, plan->threads, grid, (size_t)plan->lds_bytes, (hipStream_t)stream))
+  // c can live in LDS instead of registers when a row of the strip is one wavefront of 8-byte lanes
+  // and c's rows can be fetched 16 bytes at a time.
+  size_t lds = (size_t)plan->lds_bytes;
+  bool c_in_lds = y != nullptr && c != nullptr && es == 2 && v == 4 && plan->g_log2 == 6 && plan->steps == 8 &&
+                  (plan->threads == 256 || plan->threads == 512) && ((uintptr_t)c) % 16 == 0 &&
+                  (sc.b * es) % 16 == 0 && (sc.l * es) % 16 == 0 &&
+                  lds + fwd_c_lds_bytes(plan->threads, plan->steps) <= (size_t)kMaxLdsBytes;
+  if (c_in_lds) lds += fwd_c_lds_bytes(plan->threads, plan->steps);
+  if (!fn(args, plan->vec, plan->steps, plan->threads, c_in_lds, grid, lds, (hipStream_t)stream))
     return fail(QSSM_EINVAL, "no forward kernel for vec=%d steps=%d threads=%d", plan->vec, plan->steps, plan->threads);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : hip_fail(e, "scan_fwd_kernel launch");
@@ -408,7 +420,15 @@ int qssm_scan_backward(const qssm_plan* plan, const void* x, qssm_strides sx, co
   args.dx_sb = sdx.b; args.dx_sl = sdx.l; args.da_sb = sda.b; args.da_sl = sda.l;
   args.db_sb = sdb.b; args.db_sl = sdb.l; args.dc_sb = sdc.b; args.dc_sl = sdc.l;
   const dim3 grid((unsigned)((uint64_t)args.g.n_chains * args.g.n_seg));
-  if (!fn(args, plan->vec, plan->steps, plan->threads, grid, (size_t)plan->lds_bytes, (hipStream_t)stream))
+  // c and dy can live in LDS instead of registers when a row of the strip is one wavefront of 8-byte
+  // lanes in both and their rows can be fetched 16 bytes at a time.
+  size_t lds = (size_t)plan->lds_bytes;
+  bool cg_in_lds = es == 2 && os == 2 && v == 4 && plan->g_log2 == 6 && plan->steps == 8 && plan->threads == 256 &&
+                   ((uintptr_t)c) % 16 == 0 && (sc.b * es) % 16 == 0 && (sc.l * es) % 16 == 0 &&
+                   ((uintptr_t)dy) % 16 == 0 && (sdy.b * os) % 16 == 0 && (sdy.l * os) % 16 == 0 &&
+                   lds + bwd_cg_lds_bytes(plan->threads, plan->steps) <= (size_t)kMaxLdsBytes;
+  if (cg_in_lds) lds += bwd_cg_lds_bytes(plan->threads, plan->steps);
+  if (!fn(args, plan->vec, plan->steps, plan->threads, cg_in_lds, grid, lds, (hipStream_t)stream))
     return fail(QSSM_EINVAL, "no backward kernel for vec=%d steps=%d threads=%d", plan->vec, plan->steps, plan->threads);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : hip_fail(e, "scan_bwd_kernel launch");

@@ -20,8 +20,17 @@
 
 namespace qssm {
 
-template <typename Tin, typename Tout, int VEC, int T, int NTH>
+typedef __attribute__((address_space(1))) const void* global_ptr_t;
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// CLDS: c and dy are loaded straight into LDS (no destination registers) and read from there in the
+// sweeps that use them: 32 VGPRs fewer across the tile's whole life, which is one more resident
+// workgroup per SIMD.  Needs 64 lanes per row and 8 bytes per lane in both tensors, so that one
+// wavefront-wide 16-byte-per-lane load covers two rows of the strip.
+template <typename Tin, typename Tout, int VEC, int T, int NTH, bool CLDS>
 __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
+  static_assert(!CLDS || (sizeof(Tin) * VEC == 8 && sizeof(Tout) * VEC == 8 && T % 2 == 0),
+                "LDS-resident c and dy: 8 bytes per lane, even step count");
   extern __shared__ float lds[];
   const Geometry& g = p.g;
   const int G = 1 << g.g_log2;
@@ -35,6 +44,8 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   float* sPX = sPA + (R - 1) * cols;
   float* sE = sPX + (R - 1) * cols;      // [cols] reverse carry entering the tile
   int* sSeg = reinterpret_cast<int*>(sE + cols);
+  char* sC = reinterpret_cast<char*>(sSeg) + 16 + ((int)threadIdx.x >> 6) * (T * 512);  // CLDS: this wave's [T rows][512 bytes] of c
+  char* sG = sC + (NTH / 64) * (T * 512);                                  // and of dy
 
   const int tid = threadIdx.x;
   const int chain = blockIdx.x % g.n_chains;
@@ -95,25 +106,36 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   const unsigned long long* next_state = g.states + ((int64_t)chain * g.n_super + (s + 1)) * cols + lane;
   const bool want_map = multi && dok && j < cnt;                       // this lane group fetches the map of tile (seg + 1 + j)
   const bool want_state = multi && dok && edge && s + 1 < g.n_super;   // and the first group the next cluster's carry
-  Peek<2 * VEC> pk_map;
   Peek<VEC> pk_state;
-  pk_map.clear();
   pk_state.clear();
-  if (want_map) pk_map.issue(my_map, G);
   if (want_state) pk_state.issue(next_state, G);
 
   // ---- issue every load of the tile before touching any of them ------------------------------
-  Words<Tin, VEC> rx[T], ra[T], rb[T], rc[T];
-  Words<Tout, VEC> rg[T];
+  Words<Tin, VEC> rx[T], ra[T], rb[T], rc[CLDS ? 1 : T];
+  Words<Tout, VEC> rg[CLDS ? 1 : T];
   float hs[T][VEC];   // h(t0 + i)
   float hprev[VEC];   // h(t0 - 1); before the rebuild, the state at the tile's first step
   const bool tile_full = (t_tile + g.seg_len <= g.L) && ((strip + 1) * cols <= g.D);
   if (tile_full) {
+    if (CLDS) {
 #pragma unroll
-    for (int i = 0; i < T; ++i) {
-      ra[i] = load_stream<Tin, VEC>(ab, ao + i * as);
-      rc[i] = load_stream<Tin, VEC>(cb, co + i * cs);
-      rg[i] = load_stream<Tout, VEC>(gb, go + i * gs);
+      for (int i = 0; i < T; ++i) ra[i] = load_stream<Tin, VEC>(ab, ao + i * as);
+      // lanes 0-31 fetch one row of the strip (16 bytes each), lanes 32-63 the next one
+      const int wl = tid & 63;
+      const char* csrc = cb + (uint32_t)(j * T + (wl >> 5)) * cs + (uint32_t)(wl & 31) * 16u;
+      const char* gsrc = gb + (uint32_t)(j * T + (wl >> 5)) * gs + (uint32_t)(wl & 31) * 16u;
+#pragma unroll
+      for (int k = 0; k < T / 2; ++k) {
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(csrc + (uint32_t)(2 * k) * cs), (lds_ptr_t)(sC + k * 1024), 16, 0, 2);
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(gsrc + (uint32_t)(2 * k) * gs), (lds_ptr_t)(sG + k * 1024), 16, 0, 2);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < T; ++i) {
+        ra[i] = load_stream<Tin, VEC>(ab, ao + i * as);
+        rc[i] = load_stream<Tin, VEC>(cb, co + i * cs);
+        rg[i] = load_stream<Tout, VEC>(gb, go + i * gs);
+      }
     }
 #pragma unroll
     for (int i = 0; i < T; ++i) {
@@ -127,17 +149,36 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
       ra[i] = fill_words<Tin, VEC>(true);
       rb[i] = fill_words<Tin, VEC>(false);
       rx[i] = fill_words<Tin, VEC>(false);
-      rc[i] = fill_words<Tin, VEC>(false);
-      rg[i] = fill_words<Tout, VEC>(false);
+      if (!CLDS) {
+        rc[i] = fill_words<Tin, VEC>(false);
+        rg[i] = fill_words<Tout, VEC>(false);
+      }
     }
 #pragma unroll
     for (int i = 0; i < T; ++i) {
       if (dok && t0 + i < g.L) {
         ra[i] = load_stream<Tin, VEC>(ab, ao + i * as);
-        rc[i] = load_stream<Tin, VEC>(cb, co + i * cs);
-        rg[i] = load_stream<Tout, VEC>(gb, go + i * gs);
+        if (!CLDS) {
+          rc[i] = load_stream<Tin, VEC>(cb, co + i * cs);
+          rg[i] = load_stream<Tout, VEC>(gb, go + i * gs);
+        }
         rb[i] = load_stream<Tin, VEC>(bb, bo + i * bs);
         rx[i] = load_stream<Tin, VEC>(xb, xo + i * xs);
+      }
+    }
+    if (CLDS) {
+      // Ragged tile: c and dy go through a register one step at a time (rare, and kept rolled up so
+      // that it does not bring the registers back).
+#pragma unroll 1
+      for (int i = 0; i < T; ++i) {
+        Words<Tin, VEC> cw = fill_words<Tin, VEC>(false);
+        Words<Tout, VEC> gw = fill_words<Tout, VEC>(false);
+        if (dok && t0 + i < g.L) {
+          cw = load_stream<Tin, VEC>(cb, co + i * cs);
+          gw = load_stream<Tout, VEC>(gb, go + i * gs);
+        }
+        *reinterpret_cast<Words<Tin, VEC>*>(sC + i * 512 + (tid & 63) * 8) = cw;
+        *reinterpret_cast<Words<Tout, VEC>*>(sG + i * 512 + (tid & 63) * 8) = gw;
       }
     }
   }
@@ -168,28 +209,18 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   }
 
   // ---- the neighbours' answers (they were asked for before the operands, so they are back first)
-  pk_map.pin();
   pk_state.pin();
   bool map_here = false, state_here = false;
   float ein[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; ++v) ein[v] = 0.0f;
-  if (want_map && pk_map.ready(g.epoch)) {
-    map_here = true;
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) {
-      sPA[j * cols + dl + v] = pk_map.value(2 * v);
-      sPX[j * cols + dl + v] = pk_map.value(2 * v + 1);
-    }
-  }
   if (want_state && pk_state.ready(g.epoch)) {
     state_here = true;
 #pragma unroll
     for (int v = 0; v < VEC; ++v) ein[v] = pk_state.value(v);
   }
   // Second look for what was not there yet; the answers travel while sweep 1 runs.
-  const bool ask_map = want_map && !map_here, ask_state = want_state && !state_here;
-  if (ask_map) pk_map.issue(my_map, G);
+  const bool ask_state = want_state && !state_here;
   if (ask_state) pk_state.issue(next_state, G);
 
   // ---- sweep 1: fold this lane's T steps into the forward and the reverse affine map ----------
@@ -206,11 +237,23 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
     }
     __builtin_amdgcn_sched_barrier(0);
   }
+  // The loads that write c and dy into LDS are tracked by the vector memory counter only; this wave
+  // is the only reader of the rows it fetched.  No store of the tile has been issued yet.
+  if (CLDS) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
   for (int i = T - 1; i >= 0; --i) {
+    Words<Tin, VEC> cw;
+    Words<Tout, VEC> gw;
+    if (CLDS) {
+      cw = *reinterpret_cast<const Words<Tin, VEC>*>(sC + i * 512 + (tid & 63) * 8);
+      gw = *reinterpret_cast<const Words<Tout, VEC>*>(sG + i * 512 + (tid & 63) * 8);
+    } else {
+      cw = rc[i];
+      gw = rg[i];
+    }
 #pragma unroll
     for (int v = 0; v < VEC; ++v)
-      Xe[v] = elem(ra[i], v) * (elem(rc[i], v) * elem(rg[i], v) + Xe[v]);
+      Xe[v] = elem(ra[i], v) * (elem(cw, v) * elem(gw, v) + Xe[v]);
     __builtin_amdgcn_sched_barrier(0);
   }
 #pragma unroll
@@ -220,7 +263,10 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
     sXe[tid * VEC + v] = Xe[v];
   }
 #pragma unroll
-  for (int i = 0; i < T; ++i) { forget(ra[i]); forget(rb[i]); forget(rx[i]); forget(rc[i]); forget(rg[i]); }
+  for (int i = 0; i < T; ++i) {
+    forget(ra[i]); forget(rb[i]); forget(rx[i]);
+    if (!CLDS) { forget(rc[i]); forget(rg[i]); }
+  }
   lds_barrier();
 
   // ---- compose: groups before this one (forward state), groups after it (reverse carry) --------
@@ -269,14 +315,6 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
       }
     }
     // The second look's answers.
-    if (ask_map && pk_map.ready(g.epoch)) {
-      map_here = true;
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        sPA[j * cols + dl + v] = pk_map.value(2 * v);
-        sPX[j * cols + dl + v] = pk_map.value(2 * v + 1);
-      }
-    }
     if (ask_state && pk_state.ready(g.epoch)) {
       state_here = true;
 #pragma unroll
@@ -350,10 +388,19 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
 #pragma unroll
   for (int i = T - 1; i >= 0; --i) {
     float vdx[VEC], vda[VEC], vdb[VEC], vdc[VEC];
+    Words<Tin, VEC> cw;
+    Words<Tout, VEC> gw;
+    if (CLDS) {
+      cw = *reinterpret_cast<const Words<Tin, VEC>*>(sC + i * 512 + (tid & 63) * 8);
+      gw = *reinterpret_cast<const Words<Tout, VEC>*>(sG + i * 512 + (tid & 63) * 8);
+    } else {
+      cw = rc[i];
+      gw = rg[i];
+    }
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
-      const float gy = elem(rg[i], v);
-      const float dH = elem(rc[i], v) * gy + E[v];
+      const float gy = elem(gw, v);
+      const float dH = elem(cw, v) * gy + E[v];
       const float hm = (i == 0) ? hprev[v] : hs[i - 1][v];
       vdc[v] = gy * hs[i][v];
       vdx[v] = elem(rb[i], v) * dH;
@@ -373,26 +420,29 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
 }
 
 template <typename Tin, typename Tout>
-static bool launch_bwd(const BwdArgs& args, int vec, int steps, int threads, dim3 grid, size_t lds,
+static bool launch_bwd(const BwdArgs& args, int vec, int steps, int threads, bool cg_in_lds, dim3 grid, size_t lds,
                        hipStream_t stream) {
-#define QSSM_BWD_CASE(V, S, N)                                                                        \
-  if (vec == V && steps == S && threads == N) {                                                       \
-    hipLaunchKernelGGL((scan_bwd_kernel<Tin, Tout, V, S, N>), grid, dim3(N), lds, stream, args);       \
+#define QSSM_BWD_CASE(V, S, N, C)                                                                     \
+  if (vec == V && steps == S && threads == N && cg_in_lds == C) {                                     \
+    hipLaunchKernelGGL((scan_bwd_kernel<Tin, Tout, V, S, N, C>), grid, dim3(N), lds, stream, args);    \
     return true;                                                                                      \
   }
-  QSSM_BWD_CASE(1, 4, 256)
-  QSSM_BWD_CASE(1, 8, 256)
-  QSSM_BWD_CASE(2, 4, 256)
-  QSSM_BWD_CASE(2, 8, 256)
-  QSSM_BWD_CASE(4, 4, 256)
-  QSSM_BWD_CASE(4, 8, 256)
-  QSSM_BWD_CASE(2, 4, 512)
-  QSSM_BWD_CASE(2, 8, 512)
-  QSSM_BWD_CASE(4, 4, 512)
-  QSSM_BWD_CASE(4, 8, 512)
-  QSSM_BWD_CASE(2, 4, 1024)
-  QSSM_BWD_CASE(2, 8, 1024)
-  QSSM_BWD_CASE(4, 4, 1024)
+  if constexpr (sizeof(Tin) == 2 && sizeof(Tout) == 2) {
+    QSSM_BWD_CASE(4, 8, 256, true)
+  }
+  QSSM_BWD_CASE(1, 4, 256, false)
+  QSSM_BWD_CASE(1, 8, 256, false)
+  QSSM_BWD_CASE(2, 4, 256, false)
+  QSSM_BWD_CASE(2, 8, 256, false)
+  QSSM_BWD_CASE(4, 4, 256, false)
+  QSSM_BWD_CASE(4, 8, 256, false)
+  QSSM_BWD_CASE(2, 4, 512, false)
+  QSSM_BWD_CASE(2, 8, 512, false)
+  QSSM_BWD_CASE(4, 4, 512, false)
+  QSSM_BWD_CASE(4, 8, 512, false)
+  QSSM_BWD_CASE(2, 4, 1024, false)
+  QSSM_BWD_CASE(2, 8, 1024, false)
+  QSSM_BWD_CASE(4, 4, 1024, false)
 #undef QSSM_BWD_CASE
   return false;
 }

@@ -357,10 +357,14 @@ inline size_t bwd_lds_bytes(int nth, int vec, int cols, int cluster) {
 
 // Host-side launch tables, one entry per (in dtype, out dtype) pair the library instantiates.
 // Return false if (vec, steps, threads) is not an instantiated combination.
-typedef bool (*fwd_launch_fn)(const FwdArgs&, int vec, int steps, int threads, dim3 grid, size_t lds,
+typedef bool (*fwd_launch_fn)(const FwdArgs&, int vec, int steps, int threads, bool c_in_lds, dim3 grid, size_t lds,
                               hipStream_t stream);
-typedef bool (*bwd_launch_fn)(const BwdArgs&, int vec, int steps, int threads, dim3 grid, size_t lds,
+// Extra dynamic LDS of the forward kernel that keeps c in LDS: 8 bytes per lane and step.
+inline size_t fwd_c_lds_bytes(int nth, int steps) { return (size_t)nth * steps * 8; }
+typedef bool (*bwd_launch_fn)(const BwdArgs&, int vec, int steps, int threads, bool cg_in_lds, dim3 grid, size_t lds,
                               hipStream_t stream);
+// Extra dynamic LDS of the backward kernel that keeps c and dy in LDS.
+inline size_t bwd_cg_lds_bytes(int nth, int steps) { return (size_t)2 * nth * steps * 8; }
 
 fwd_launch_fn find_fwd_launcher(int in_dtype, int out_dtype);
 bwd_launch_fn find_bwd_launcher(int in_dtype, int out_dtype);

@@ -10,8 +10,16 @@
 
 namespace qssm {
 
-template <typename Tin, typename Tout, int VEC, int T, int NTH>
+typedef __attribute__((address_space(1))) const void* global_ptr_t;
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// CLDS: the c operand is not needed before the last sweep, so it is loaded straight into LDS
+// (no destination registers) and read from there step by step: 16 VGPRs fewer across the
+// tile's whole life, which is one more resident workgroup per SIMD.  Needs 64 lanes per row and
+// 8 bytes per lane, so that one wavefront-wide 16-byte-per-lane load covers two rows of the strip.
+template <typename Tin, typename Tout, int VEC, int T, int NTH, bool CLDS>
 __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
+  static_assert(!CLDS || (sizeof(Tin) * VEC == 8 && T % 2 == 0), "LDS-resident c: 8 bytes per lane, even step count");
   extern __shared__ float lds[];
   const Geometry& g = p.g;
   const int G = 1 << g.g_log2;
@@ -24,6 +32,7 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   float* sPX = sPA + (R - 1) * cols;
   float* sH = sPX + (R - 1) * cols;      // [cols] state entering the tile
   int* sSeg = reinterpret_cast<int*>(sH + cols);
+  char* sC = reinterpret_cast<char*>(sSeg) + 16;  // CLDS: [NTH / 64 waves][T rows][512 bytes] of c
 
   const int tid = threadIdx.x;
   const int chain = blockIdx.x % g.n_chains;
@@ -95,7 +104,7 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   if (want_state) pk_state.issue(prev_state, G);
 
   // ---- issue every load of the tile before touching any of them ------------------------------
-  Words<Tin, VEC> rx[T], ra[T], rb[T], rc[T];
+  Words<Tin, VEC> rx[T], ra[T], rb[T], rc[CLDS ? 1 : T];
   const bool tile_full = (t_tile + g.seg_len <= g.L) && ((strip + 1) * cols <= g.D);
   if (tile_full) {
 #pragma unroll
@@ -104,7 +113,15 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
       rb[i] = load_stream<Tin, VEC>(bb, bo + i * bs);
       rx[i] = load_stream<Tin, VEC>(xb, xo + i * xs);
     }
-    if (has_c) {
+    if (CLDS) {
+      // lanes 0-31 fetch one row of the strip (16 bytes each), lanes 32-63 the next one
+      const int wl = tid & 63;
+      const char* src = cb + (uint32_t)(j * T + (wl >> 5)) * cs + (uint32_t)(wl & 31) * 16u;
+      char* dst = sC + (tid >> 6) * (T * 512);
+#pragma unroll
+      for (int k = 0; k < T / 2; ++k)
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(src + (uint32_t)(2 * k) * cs), (lds_ptr_t)(dst + k * 1024), 16, 0, 2);
+    } else if (has_c) {
 #pragma unroll
       for (int i = 0; i < T; ++i) rc[i] = load_stream<Tin, VEC>(cb, co + i * cs);
     }
@@ -115,7 +132,7 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
       ra[i] = fill_words<Tin, VEC>(true);
       rb[i] = fill_words<Tin, VEC>(false);
       rx[i] = fill_words<Tin, VEC>(false);
-      rc[i] = fill_words<Tin, VEC>(false);
+      if (!CLDS) rc[i] = fill_words<Tin, VEC>(false);
     }
 #pragma unroll
     for (int i = 0; i < T; ++i) {
@@ -123,7 +140,18 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
         ra[i] = load_stream<Tin, VEC>(ab, ao + i * as);
         rb[i] = load_stream<Tin, VEC>(bb, bo + i * bs);
         rx[i] = load_stream<Tin, VEC>(xb, xo + i * xs);
-        if (has_c) rc[i] = load_stream<Tin, VEC>(cb, co + i * cs);
+        if (!CLDS && has_c) rc[i] = load_stream<Tin, VEC>(cb, co + i * cs);
+      }
+    }
+    if (CLDS) {
+      // Ragged tile: c goes through a register one step at a time (rare, and kept rolled up so that
+      // it does not bring the sixteen registers back).
+      char* dst = sC + (tid >> 6) * (T * 512) + (tid & 63) * 8;
+#pragma unroll 1
+      for (int i = 0; i < T; ++i) {
+        Words<Tin, VEC> cw = fill_words<Tin, VEC>(false);
+        if (dok && t0 + i < g.L) cw = load_stream<Tin, VEC>(cb, co + i * cs);
+        *reinterpret_cast<Words<Tin, VEC>*>(dst + i * 512) = cw;
       }
     }
   }
@@ -177,6 +205,10 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   QSSM_STAMP(1);
   lds_barrier();
   QSSM_STAMP(2);
+  // The loads that write c into LDS are tracked by the vector memory counter only; this wave is the
+  // only reader of the rows it fetched.  Waiting here, before any store of the tile is issued, waits
+  // for nothing but loads.
+  if (CLDS) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   // ---- compose the maps of the lane groups before this one ------------------------------------
   float Ap[VEC], Xp[VEC];
@@ -288,10 +320,13 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
 #pragma unroll
   for (int i = 0; i < T; ++i) {
     float yv[VEC];
+    Words<Tin, VEC> cw;
+    if (CLDS) cw = *reinterpret_cast<const Words<Tin, VEC>*>(sC + (tid >> 6) * (T * 512) + i * 512 + (tid & 63) * 8);
+    else cw = rc[i];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
       h[v] = elem(ra[i], v) * h[v] + elem(rb[i], v) * elem(rx[i], v);
-      yv[v] = has_c ? elem(rc[i], v) * h[v] : h[v];
+      yv[v] = (CLDS || has_c) ? elem(cw, v) * h[v] : h[v];
     }
     if (tile_full || (dok && t0 + i < g.L)) {
       if (want_y) store_stream<Tout, VEC>(yb, yo + i * ys, yv);
@@ -305,27 +340,31 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
 }
 
 template <typename Tin, typename Tout>
-static bool launch_fwd(const FwdArgs& args, int vec, int steps, int threads, dim3 grid, size_t lds,
+static bool launch_fwd(const FwdArgs& args, int vec, int steps, int threads, bool c_in_lds, dim3 grid, size_t lds,
                        hipStream_t stream) {
-#define QSSM_FWD_CASE(V, S, N)                                                                        \
-  if (vec == V && steps == S && threads == N) {                                                       \
-    hipLaunchKernelGGL((scan_fwd_kernel<Tin, Tout, V, S, N>), grid, dim3(N), lds, stream, args);       \
+#define QSSM_FWD_CASE(V, S, N, C)                                                                     \
+  if (vec == V && steps == S && threads == N && c_in_lds == C) {                                      \
+    hipLaunchKernelGGL((scan_fwd_kernel<Tin, Tout, V, S, N, C>), grid, dim3(N), lds, stream, args);    \
     return true;                                                                                      \
   }
-  QSSM_FWD_CASE(1, 4, 256)
-  QSSM_FWD_CASE(1, 8, 256)
-  QSSM_FWD_CASE(2, 4, 256)
-  QSSM_FWD_CASE(2, 8, 256)
-  QSSM_FWD_CASE(4, 4, 256)
-  QSSM_FWD_CASE(4, 8, 256)
-  QSSM_FWD_CASE(2, 4, 512)
-  QSSM_FWD_CASE(2, 8, 512)
-  QSSM_FWD_CASE(4, 4, 512)
-  QSSM_FWD_CASE(4, 8, 512)
-  QSSM_FWD_CASE(2, 4, 1024)
-  QSSM_FWD_CASE(2, 8, 1024)
-  QSSM_FWD_CASE(4, 4, 1024)
-  QSSM_FWD_CASE(4, 8, 1024)
+  if constexpr (sizeof(Tin) == 2) {
+    QSSM_FWD_CASE(4, 8, 256, true)
+    QSSM_FWD_CASE(4, 8, 512, true)
+  }
+  QSSM_FWD_CASE(1, 4, 256, false)
+  QSSM_FWD_CASE(1, 8, 256, false)
+  QSSM_FWD_CASE(2, 4, 256, false)
+  QSSM_FWD_CASE(2, 8, 256, false)
+  QSSM_FWD_CASE(4, 4, 256, false)
+  QSSM_FWD_CASE(4, 8, 256, false)
+  QSSM_FWD_CASE(2, 4, 512, false)
+  QSSM_FWD_CASE(2, 8, 512, false)
+  QSSM_FWD_CASE(4, 4, 512, false)
+  QSSM_FWD_CASE(4, 8, 512, false)
+  QSSM_FWD_CASE(2, 4, 1024, false)
+  QSSM_FWD_CASE(2, 8, 1024, false)
+  QSSM_FWD_CASE(4, 4, 1024, false)
+  QSSM_FWD_CASE(4, 8, 1024, false)
 #undef QSSM_FWD_CASE
   return false;
 }

@@ -80,8 +80,8 @@ def _ptr(t: Optional[Tensor]) -> Optional[int]:
 
 
 def _align_elems(tensors: Sequence[Optional[Tensor]], D: int) -> int:
-    """Largest v in (4, 2, 1) such that D, every stride and every base address (in elements) divide by v."""
-    for v in (4, 2):
+    """Largest v in (8, 4, 2, 1) such that D, every stride and every base address (in elements) divide by v."""
+    for v in (8, 4, 2):
         ok = D % v == 0
         for t in tensors:
             if not ok:
