@@ -31,7 +31,7 @@ template <typename Tin, typename Tout, int VEC, int T, int NTH, bool CLDS>
 __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   static_assert(!CLDS || (sizeof(Tin) * VEC == 8 && sizeof(Tout) * VEC == 8 && T % 2 == 0),
                 "LDS-resident c and dy: 8 bytes per lane, even step count");
-  extern __shared__ float lds[];
+  extern __shared__ __align__(16) float lds[];
   const Geometry& g = p.g;
   const int G = 1 << g.g_log2;
   const int NG = NTH >> g.g_log2;
@@ -53,13 +53,9 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   // ---- claim a tile of this chain, last tile in time first -----------------------------------
   int seg = 0;
   if (g.n_seg > 1) {
-#ifdef QSSM_PROBE_STATIC
-    const int tk = blockIdx.x / g.n_chains;
-#else
     if (tid == 0) *sSeg = (int)claim_ticket(g.tickets, chain, g.n_seg);
     __syncthreads();
     const int tk = __builtin_amdgcn_readfirstlane(*sSeg);
-#endif
     if ((unsigned)tk >= (unsigned)g.n_seg) {  // the control block was not zero on entry
       if (tid == 0) raise_status(g.status, 2);
       return;
@@ -91,11 +87,7 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   const float* hp = p.h + (int64_t)bi * p.h_sb + (int64_t)t0 * p.h_sl + d;
 
   // ---- ask for the neighbours' words first: they are looked at once the answers are back ------
-#ifdef QSSM_PROBE_NOCHAIN
-  const bool multi = false;
-#else
   const bool multi = g.n_seg > 1;
-#endif
   const int s = seg / R;                                     // cluster of this tile
   const int m = seg - s * R;                                 // tiles of the cluster before this one
   const int last = ((s + 1) * R < g.n_seg ? (s + 1) * R : g.n_seg) - 1;
@@ -256,12 +248,9 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
       Xe[v] = elem(ra[i], v) * (elem(cw, v) * elem(gw, v) + Xe[v]);
     __builtin_amdgcn_sched_barrier(0);
   }
-#pragma unroll
-  for (int v = 0; v < VEC; ++v) {
-    sA[tid * VEC + v] = A[v];
-    sXf[tid * VEC + v] = Xf[v];
-    sXe[tid * VEC + v] = Xe[v];
-  }
+  lds_put<VEC>(sA + tid * VEC, A);
+  lds_put<VEC>(sXf + tid * VEC, Xf);
+  lds_put<VEC>(sXe + tid * VEC, Xe);
 #pragma unroll
   for (int i = 0; i < T; ++i) {
     forget(ra[i]); forget(rb[i]); forget(rx[i]);
@@ -276,21 +265,25 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   if (!have_h) {
 #pragma unroll 4
     for (int k = 0; k < j; ++k) {
+      float ak[VEC], xk[VEC];
+      lds_get<VEC>(sA + k * cols + dl, ak);
+      lds_get<VEC>(sXf + k * cols + dl, xk);
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
-        const float ak = sA[k * cols + dl + v];
-        Xp[v] = ak * Xp[v] + sXf[k * cols + dl + v];
-        Ap[v] = ak * Ap[v];
+        Xp[v] = ak[v] * Xp[v] + xk[v];
+        Ap[v] = ak[v] * Ap[v];
       }
     }
   }
 #pragma unroll 4
   for (int k = NG - 1; k > j; --k) {
+    float ak[VEC], xk[VEC];
+    lds_get<VEC>(sA + k * cols + dl, ak);
+    lds_get<VEC>(sXe + k * cols + dl, xk);
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
-      const float ak = sA[k * cols + dl + v];
-      Xs[v] = ak * Xs[v] + sXe[k * cols + dl + v];
-      As[v] = ak * As[v];
+      Xs[v] = ak[v] * Xs[v] + xk[v];
+      As[v] = ak[v] * As[v];
     }
   }
 
@@ -298,11 +291,13 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   if (multi) {
     float At[VEC], Xt[VEC];
     if (edge) {
+      float av[VEC], xv[VEC];
+      lds_get<VEC>(sA + tid * VEC, av);
+      lds_get<VEC>(sXe + tid * VEC, xv);
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
-        const float av = sA[tid * VEC + v];
-        At[v] = av * As[v];
-        Xt[v] = av * Xs[v] + sXe[tid * VEC + v];
+        At[v] = av[v] * As[v];
+        Xt[v] = av[v] * Xs[v] + xv[v];
       }
       // Earlier tiles of the cluster need this tile's map; it depends on nothing, so it goes out first.
       if (dok && m > 0) {
@@ -327,34 +322,35 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
       if (dok && !(i == j && map_here)) {
         float w[2 * VEC];
         const unsigned long long* mw = g.maps + ((int64_t)chain * g.n_seg + (seg + 1 + i)) * cols * 2 + lane;
-        if (!words_wait<2 * VEC, false>(mw, G, g.epoch, w)) raise_status(g.status, 1);
+        if (!words_wait<2 * VEC>(mw, G, g.epoch, w, kPollSlow)) raise_status(g.status, 1);
+        float wa[VEC], wx[VEC];
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) {
-          sPA[i * cols + dl + v] = w[2 * v];
-          sPX[i * cols + dl + v] = w[2 * v + 1];
-        }
+        for (int v = 0; v < VEC; ++v) { wa[v] = w[2 * v]; wx[v] = w[2 * v + 1]; }
+        lds_put<VEC>(sPA + i * cols + dl, wa);
+        lds_put<VEC>(sPX + i * cols + dl, wx);
       }
     }
     if (want_state && !state_here) {
-      if (!words_wait<VEC, true>(next_state, G, g.epoch, ein)) raise_status(g.status, 1);
+      if (!words_wait<VEC>(next_state, G, g.epoch, ein, m == 0 ? kPollChain : kPollUrgent)) raise_status(g.status, 1);
     }
     if (cnt > 0) lds_barrier();
     if (edge) {
       for (int i = cnt - 1; i >= 0; --i) {
+        float pa[VEC], px[VEC];
+        lds_get<VEC>(sPA + i * cols + dl, pa);
+        lds_get<VEC>(sPX + i * cols + dl, px);
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) ein[v] = sPA[i * cols + dl + v] * ein[v] + sPX[i * cols + dl + v];
+        for (int v = 0; v < VEC; ++v) ein[v] = pa[v] * ein[v] + px[v];
       }
       if (dok && m == 0 && s > 0) {
         unsigned long long* sw = g.states + ((int64_t)chain * g.n_super + s) * cols + lane;
 #pragma unroll
         for (int v = 0; v < VEC; ++v) word_publish(sw + v * G, g.epoch, At[v] * ein[v] + Xt[v]);
       }
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) sE[dl + v] = ein[v];
+      lds_put<VEC>(sE + dl, ein);
     }
     lds_barrier();
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) ein[v] = sE[dl + v];
+    lds_get<VEC>(sE + dl, ein);
   }
 
   float E[VEC];

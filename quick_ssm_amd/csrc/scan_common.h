@@ -106,11 +106,13 @@ template <> struct ElemBits<bf16_t> {
     if (V == 1) {
       p.w[0] = (uint32_t)__builtin_bit_cast(unsigned short, (bf16_t)f[0]);
     } else {
+      // two values per conversion instruction, already packed
+      typedef float f32x2 __attribute__((ext_vector_type(2)));
+      typedef bf16_t bf16x2 __attribute__((ext_vector_type(2)));
 #pragma unroll
       for (int k = 0; k < V / 2; ++k) {
-        const uint32_t lo = __builtin_bit_cast(unsigned short, (bf16_t)f[2 * k]);
-        const uint32_t hi = __builtin_bit_cast(unsigned short, (bf16_t)f[2 * k + 1]);
-        p.w[k] = lo | (hi << 16);
+        const f32x2 pair = {f[2 * k], f[2 * k + 1]};
+        p.w[k] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
       }
     }
   }
@@ -196,6 +198,23 @@ __device__ __forceinline__ void store_pack(T* p, const Pack<T, V>& v) {
   *reinterpret_cast<raw_t*>(p) = __builtin_bit_cast(raw_t, v);
 }
 
+// VEC adjacent floats in LDS as one access (a lane's VEC columns sit next to each other, so a
+// wavefront's access is dense and free of bank conflicts, which VEC separate 4-byte accesses at a
+// stride of VEC words are not).
+template <int V>
+__device__ __forceinline__ void lds_get(const float* p, float* out) {
+  const Pack<float, V> v = *reinterpret_cast<const Pack<float, V>*>(p);
+#pragma unroll
+  for (int k = 0; k < V; ++k) out[k] = v.v[k];
+}
+template <int V>
+__device__ __forceinline__ void lds_put(float* p, const float* in) {
+  Pack<float, V> v;
+#pragma unroll
+  for (int k = 0; k < V; ++k) v.v[k] = in[k];
+  *reinterpret_cast<Pack<float, V>*>(p) = v;
+}
+
 // Makes the compiler forget what it knows about a loaded operand, so that the later sweeps
 // convert it to fp32 again instead of keeping an fp32 copy of every operand alive across the
 // barriers (which would double the register footprint of a tile).
@@ -255,26 +274,27 @@ struct Peek {
   __device__ __forceinline__ float value(int n) const { return __uint_as_float((unsigned)r[n]); }
 };
 
-// Wait until this lane's N words (at w + n * plane) carry this launch's epoch.  While waiting, a
-// wavefront polls ONE word (its first active lane's first word, read by every lane at the same
-// address, i.e. one 8-byte request); only when that one has arrived do the lanes read their own
-// words, which the producer stored with the same instructions and which are then there as a rule.
-// This keeps a waiting tile's traffic at a few bytes per poll instead of a full row of words.
-// Returns false (and NaN payloads) if the words never arrive.
-template <int N, bool URGENT>
-__device__ __forceinline__ bool words_wait(const unsigned long long* w, int plane, unsigned epoch, float* out) {
-  const uint64_t mine = reinterpret_cast<uint64_t>(w);
-  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)mine);
-  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(mine >> 32));
-  unsigned long long* lead = reinterpret_cast<unsigned long long*>(((uint64_t)hi << 32) | lo);
-  // URGENT: the hand-over between clusters is the one serial path of the whole launch, so that
-  // waiter polls almost back to back at first and backs off (to about half a microsecond between
-  // polls) only when the wait drags on.  Everything else is needed later than it is published as
-  // a rule, and is polled at the slow rate from the start, so that waiting tiles do not load the
-  // memory system.
-  for (int spins = 0; spins < kSpinLimit; ++spins) {
-    const unsigned long long first = __hip_atomic_load(lead, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if ((unsigned)(first >> 32) == epoch) {
+// Wait until this lane's N words (at w + n * plane) carry this launch's epoch.  Returns false (and
+// NaN payloads) if the words never arrive.  Three ways of polling:
+//   kPollSlow    one word per wavefront (its first active lane's first word, read by every lane at
+//                the same address, i.e. one 8-byte request), about half a microsecond apart; only
+//                when that one has arrived do the lanes read their own words, which the producer
+//                stored with the same instructions and which are then there as a rule.  For words
+//                that are needed later than they are published as a rule: a waiting tile must not
+//                load the memory system.
+//   kPollUrgent  the same, almost back to back at first, backing off when the wait drags on.  For
+//                the state a tile needs but does not hand on.
+//   kPollChain   every lane polls its own words, back to back: the answer that shows the words is
+//                the answer that carries them, which saves a round trip per hand-over.  Only for the
+//                one tile per cluster that hands the state on, i.e. one waiting tile per chain: the
+//                hand-overs from cluster to cluster are the serial path of the whole launch.
+enum PollMode { kPollSlow = 0, kPollUrgent = 1, kPollChain = 2 };
+
+template <int N>
+__device__ __forceinline__ bool words_wait(const unsigned long long* w, int plane, unsigned epoch, float* out,
+                                           const PollMode mode) {
+  if (mode == kPollChain) {
+    for (int spins = 0; spins < kSpinLimit; ++spins) {
       Peek<N> pk;
       pk.issue(w, plane);
       if (pk.ready(epoch)) {
@@ -282,12 +302,33 @@ __device__ __forceinline__ bool words_wait(const unsigned long long* w, int plan
         for (int n = 0; n < N; ++n) out[n] = pk.value(n);
         return true;
       }
+      if (spins >= 64) {
+        for (int k = 0; k < 8; ++k) __builtin_amdgcn_s_sleep(2);
+      }
     }
-    if (URGENT && spins < 32) {
-      __builtin_amdgcn_s_sleep(1);
-    } else {
-      const int nap = (URGENT && spins < 256) ? 2 : 8;
-      for (int k = 0; k < nap; ++k) __builtin_amdgcn_s_sleep(2);
+  } else {
+    const uint64_t mine = reinterpret_cast<uint64_t>(w);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)mine);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(mine >> 32));
+    unsigned long long* lead = reinterpret_cast<unsigned long long*>(((uint64_t)hi << 32) | lo);
+    const bool urgent = mode == kPollUrgent;
+    for (int spins = 0; spins < kSpinLimit; ++spins) {
+      const unsigned long long first = __hip_atomic_load(lead, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if ((unsigned)(first >> 32) == epoch) {
+        Peek<N> pk;
+        pk.issue(w, plane);
+        if (pk.ready(epoch)) {
+#pragma unroll
+          for (int n = 0; n < N; ++n) out[n] = pk.value(n);
+          return true;
+        }
+      }
+      if (urgent && spins < 32) {
+        __builtin_amdgcn_s_sleep(1);
+      } else {
+        const int nap = (urgent && spins < 256) ? 2 : 8;
+        for (int k = 0; k < nap; ++k) __builtin_amdgcn_s_sleep(2);
+      }
     }
   }
 #pragma unroll

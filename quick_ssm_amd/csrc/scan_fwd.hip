@@ -6,6 +6,8 @@
 // quick_ssm/triton_forwards.py:33-131) and of the y = c*h multiply and cast that follow them
 // (quick_ssm/scan_interface.py:104-107).  The affine-map composition is the reference's
 // combine_fn (quick_ssm/triton_forwards.py:26-30): (aL,xL) then (aR,xR) = (aR*aL, aR*xL+xR).
+#include <type_traits>
+
 #include "scan_common.h"
 
 namespace qssm {
@@ -20,7 +22,7 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 template <typename Tin, typename Tout, int VEC, int T, int NTH, bool CLDS>
 __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   static_assert(!CLDS || (sizeof(Tin) * VEC == 8 && T % 2 == 0), "LDS-resident c: 8 bytes per lane, even step count");
-  extern __shared__ float lds[];
+  extern __shared__ __align__(16) float lds[];
   const Geometry& g = p.g;
   const int G = 1 << g.g_log2;
   const int NG = NTH >> g.g_log2;
@@ -40,26 +42,15 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   // ---- claim a tile of this chain, in time order -------------------------------------------
   int seg = 0;
   if (g.n_seg > 1) {
-#ifdef QSSM_PROBE_STATIC
-    seg = blockIdx.x / g.n_chains;
-#else
     if (tid == 0) *sSeg = (int)claim_ticket(g.tickets, chain, g.n_seg);
     __syncthreads();
     seg = __builtin_amdgcn_readfirstlane(*sSeg);
-#endif
     if ((unsigned)seg >= (unsigned)g.n_seg) {  // the control block was not zero on entry
       if (tid == 0) raise_status(g.status, 2);
       return;
     }
   }
 
-#ifdef QSSM_PROBE_TIMELINE
-  unsigned long long* stamps = g.states + (int64_t)g.n_chains * g.n_super * (G * VEC) + ((int64_t)chain * g.n_seg + seg) * 8;
-#define QSSM_STAMP(k) do { if (tid == NTH - 1) stamps[k] = wall_clock64(); } while (0)
-  QSSM_STAMP(0);
-#else
-#define QSSM_STAMP(k) do {} while (0)
-#endif
   const int bi = chain / g.n_strips;
   const int strip = chain - bi * g.n_strips;
   const int j = tid >> g.g_log2;         // lane group = time sub-segment
@@ -83,11 +74,7 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   const bool has_c = want_y && p.c != nullptr;
 
   // ---- ask for the neighbours' words first: they are looked at once the answers are back ------
-#ifdef QSSM_PROBE_NOCHAIN
-  const bool multi = false;
-#else
   const bool multi = g.n_seg > 1;
-#endif
   const int s = seg / R;               // cluster of this tile
   const int m = seg - s * R;           // tiles of the cluster before this one
   const bool edge = (j == NG - 1);     // the last lane group holds the tile's total map
@@ -165,11 +152,11 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   for (int v = 0; v < VEC; ++v) hin[v] = 0.0f;
   if (want_map && pk_map.ready(g.epoch)) {
     map_here = true;
+    float wa[VEC], wx[VEC];
 #pragma unroll
-    for (int v = 0; v < VEC; ++v) {
-      sPA[j * cols + dl + v] = pk_map.value(2 * v);
-      sPX[j * cols + dl + v] = pk_map.value(2 * v + 1);
-    }
+    for (int v = 0; v < VEC; ++v) { wa[v] = pk_map.value(2 * v); wx[v] = pk_map.value(2 * v + 1); }
+    lds_put<VEC>(sPA + j * cols + dl, wa);
+    lds_put<VEC>(sPX + j * cols + dl, wx);
   }
   if (want_state && pk_state.ready(g.epoch)) {
     state_here = true;
@@ -195,16 +182,11 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
     }
     __builtin_amdgcn_sched_barrier(0);
   }
-#pragma unroll
-  for (int v = 0; v < VEC; ++v) {
-    sA[tid * VEC + v] = A[v];
-    sX[tid * VEC + v] = X[v];
-  }
+  lds_put<VEC>(sA + tid * VEC, A);
+  lds_put<VEC>(sX + tid * VEC, X);
 #pragma unroll
   for (int i = 0; i < T; ++i) { forget(ra[i]); forget(rb[i]); forget(rx[i]); }
-  QSSM_STAMP(1);
   lds_barrier();
-  QSSM_STAMP(2);
   // The loads that write c into LDS are tracked by the vector memory counter only; this wave is the
   // only reader of the rows it fetched.  Waiting here, before any store of the tile is issued, waits
   // for nothing but loads.
@@ -216,11 +198,13 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   for (int v = 0; v < VEC; ++v) { Ap[v] = 1.0f; Xp[v] = 0.0f; }
 #pragma unroll 4
   for (int k = 0; k < j; ++k) {
+    float ak[VEC], xk[VEC];
+    lds_get<VEC>(sA + k * cols + dl, ak);
+    lds_get<VEC>(sX + k * cols + dl, xk);
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
-      const float ak = sA[k * cols + dl + v];
-      Xp[v] = ak * Xp[v] + sX[k * cols + dl + v];
-      Ap[v] = ak * Ap[v];
+      Xp[v] = ak[v] * Xp[v] + xk[v];
+      Ap[v] = ak[v] * Ap[v];
     }
   }
 
@@ -228,11 +212,13 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   if (multi) {
     float At[VEC], Xt[VEC];
     if (edge) {
+      float av[VEC], xv[VEC];
+      lds_get<VEC>(sA + tid * VEC, av);
+      lds_get<VEC>(sX + tid * VEC, xv);
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
-        const float av = sA[tid * VEC + v];
-        At[v] = av * Ap[v];
-        Xt[v] = av * Xp[v] + sX[tid * VEC + v];
+        At[v] = av[v] * Ap[v];
+        Xt[v] = av[v] * Xp[v] + xv[v];
       }
       // Later tiles of the cluster need this tile's map; it depends on nothing, so it goes out first.
       if (dok && m + 1 < R && seg + 1 < g.n_seg) {
@@ -247,11 +233,11 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
     // The second look's answers.
     if (ask_map && pk_map.ready(g.epoch)) {
       map_here = true;
+      float wa[VEC], wx[VEC];
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        sPA[j * cols + dl + v] = pk_map.value(2 * v);
-        sPX[j * cols + dl + v] = pk_map.value(2 * v + 1);
-      }
+      for (int v = 0; v < VEC; ++v) { wa[v] = pk_map.value(2 * v); wx[v] = pk_map.value(2 * v + 1); }
+      lds_put<VEC>(sPA + j * cols + dl, wa);
+      lds_put<VEC>(sPX + j * cols + dl, wx);
     }
     if (ask_state && pk_state.ready(g.epoch)) {
       state_here = true;
@@ -265,39 +251,36 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
       if (dok && !(i == j && map_here)) {
         float w[2 * VEC];
         const unsigned long long* mw = g.maps + ((int64_t)chain * g.n_seg + (seg - m + i)) * cols * 2 + lane;
-        if (!words_wait<2 * VEC, false>(mw, G, g.epoch, w)) raise_status(g.status, 1);
+        if (!words_wait<2 * VEC>(mw, G, g.epoch, w, kPollSlow)) raise_status(g.status, 1);
+        float wa[VEC], wx[VEC];
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) {
-          sPA[i * cols + dl + v] = w[2 * v];
-          sPX[i * cols + dl + v] = w[2 * v + 1];
-        }
+        for (int v = 0; v < VEC; ++v) { wa[v] = w[2 * v]; wx[v] = w[2 * v + 1]; }
+        lds_put<VEC>(sPA + i * cols + dl, wa);
+        lds_put<VEC>(sPX + i * cols + dl, wx);
       }
     }
-    QSSM_STAMP(3);
     if (want_state && !state_here) {
-      if (!words_wait<VEC, true>(prev_state, G, g.epoch, hin)) raise_status(g.status, 1);
+      if (!words_wait<VEC>(prev_state, G, g.epoch, hin, m == R - 1 ? kPollChain : kPollUrgent)) raise_status(g.status, 1);
     }
-    QSSM_STAMP(4);
     if (m > 0) lds_barrier();
-    QSSM_STAMP(5);
     if (edge) {
       for (int i = 0; i < m; ++i) {
+        float pa[VEC], px[VEC];
+        lds_get<VEC>(sPA + i * cols + dl, pa);
+        lds_get<VEC>(sPX + i * cols + dl, px);
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) hin[v] = sPA[i * cols + dl + v] * hin[v] + sPX[i * cols + dl + v];
+        for (int v = 0; v < VEC; ++v) hin[v] = pa[v] * hin[v] + px[v];
       }
       if (dok && m == R - 1 && s + 1 < g.n_super) {
         unsigned long long* sw = g.states + ((int64_t)chain * g.n_super + s) * cols + lane;
 #pragma unroll
         for (int v = 0; v < VEC; ++v) word_publish(sw + v * G, g.epoch, At[v] * hin[v] + Xt[v]);
       }
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) sH[dl + v] = hin[v];
+      lds_put<VEC>(sH + dl, hin);
     }
     lds_barrier();
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) hin[v] = sH[dl + v];
+    lds_get<VEC>(sH + dl, hin);
   }
-  QSSM_STAMP(6);
 
   float h[VEC];
 #pragma unroll
@@ -336,7 +319,6 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
     // would hold an fp32 copy of the whole tile in registers.
     __builtin_amdgcn_sched_barrier(0);
   }
-  QSSM_STAMP(7);
 }
 
 template <typename Tin, typename Tout>
