@@ -13,7 +13,7 @@ import torch
 
 import oracle
 from helpers import TOL, assert_close, make_inputs, oracle_all, run_scan_with_grads
-from quick_ssm_amd import hip_scan
+from quick_ssm_amd import _lib, hip_scan
 from quick_ssm_amd.scan_interface import honor_tiles, scan
 
 pytestmark = pytest.mark.gpu
@@ -105,6 +105,8 @@ SHAPES = [
     (1, 4096, 128),
     (2, 1500, 260),   # two strips, the second partial
     (5, 64, 1024),    # config 4's per-layer shape (smaller batch)
+    (2, 1100, 264),   # 16-bit: operands through LDS, ragged last tile, second strip of 8 columns
+    (3, 200, 512),    # 16-bit: operands through LDS, whole strips, short ragged sequence
 ]
 
 
@@ -129,6 +131,55 @@ def test_fp32_output_from_16bit_operands(gpu, dtype):
     assert_close("y", got["y"], ref["y"], 1e-5)  # fp32 storage of y: only fp32 arithmetic error remains
     for k in ("dx", "da", "db", "dc"):
         assert_close(k, got[k], ref[k], TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+@pytest.mark.parametrize("shape", [(2, 700, 512), (2, 1100, 264), (1, 97, 256)], ids=lambda s: "x".join(map(str, s)))
+def test_lds_resident_operands_and_register_path_agree(gpu, dtype, shape):
+    # 64-lane rows whose bytes are 16-byte aligned take the kernels that load c (and dy) straight into LDS; the
+    # same values at an offset of 4 elements take the register-only kernels.  Both must meet the oracle: ragged last
+    # tiles, a partial second strip, checkpoint on and off, y in the operands' storage and in fp32.
+    B, L, D = shape
+    x, a, b, c, dy = make_inputs(shape, dtype=dtype, seed=31)
+    ref = oracle_all(x, a, b, c, dy)
+    tune = 7 | (8 << 8)  # 64 lanes per row, 8 steps per lane; workgroup size and clusters automatic
+
+    def run(place, out_dtype=dtype, gy=dy, keep_h=False):
+        ops = [place(t) for t in (x, a, b, c)]
+        g = place(gy)
+        y, h, ckpt, stride = hip_scan.scan_forward(*ops, out_dtype=out_dtype, want_h=keep_h, want_ckpt=not keep_h,
+                                                   tune=tune, bwd_tune=tune)
+        dx, da, db, dc = hip_scan.scan_backward(*ops, g, h=h, ckpt=ckpt, ckpt_stride=stride, tune=tune)
+        assert hip_scan.workspace_status() == 0
+        return {k: v.cpu() for k, v in zip(("y", "dx", "da", "db", "dc"), (y, dx, da, db, dc))}, ops
+
+    def aligned(t):
+        return t.to(gpu).contiguous()
+
+    def shifted(t):  # same values, every row 8 bytes (4 elements) off a 16-byte boundary
+        buf = torch.zeros(B, L, D + 8, dtype=t.dtype, device=gpu)
+        buf[:, :, 4:4 + D] = t.to(gpu)
+        return buf[:, :, 4:4 + D]
+
+    got_lds, ops = run(aligned)
+    assert all(t.data_ptr() % 16 == 0 for t in ops)
+    fwd_plan = hip_scan.make_plan(B, L, D, dtype, dtype, _lib.QSSM_FORWARD, 8, 32, tune)
+    bwd_plan = hip_scan.make_plan(B, L, D, dtype, dtype, _lib.QSSM_BACKWARD, 8, 0, tune)
+    assert (fwd_plan.g_log2, fwd_plan.vec, fwd_plan.steps) == (6, 4, 8) and fwd_plan.threads in (256, 512)
+    assert (bwd_plan.g_log2, bwd_plan.vec, bwd_plan.steps, bwd_plan.threads) == (6, 4, 8, 256)
+    _check_all(got_lds, ref, TOL[dtype])
+    _check_all(run(aligned, keep_h=True)[0], ref, TOL[dtype])
+
+    got_reg, ops = run(shifted)
+    assert all(t.data_ptr() % 16 == 8 for t in ops) and D % 8 == 0
+    _check_all(got_reg, ref, TOL[dtype])
+
+    x32, a32, b32, c32, dy32 = make_inputs(shape, dtype=dtype, seed=31, out_dtype=torch.float32)
+    got32, _ = run(aligned, out_dtype=torch.float32, gy=dy32)   # forward through LDS, backward (fp32 dy) not
+    ref32 = oracle_all(x32, a32, b32, c32, dy32)
+    assert_close("y", got32["y"], ref32["y"], 1e-5)
+    for k in ("dx", "da", "db", "dc"):
+        assert_close(k, got32[k], ref32[k], TOL[dtype])
 
 
 def test_mixed_operand_dtypes_and_unbuilt_output_dtype(gpu):
