@@ -165,6 +165,30 @@ QSSM_API int qssm_scan_forward(const qssm_plan* plan,
                       void* stream);
 
 /*
+ * Forward scan with a carried state: the same launch, started from `h_init` instead of zero and/or
+ * reporting the state after the last step, so that a sequence can be scanned in pieces (chunked
+ * prefill, token-by-token generation) with results identical to one scan over the whole of it.
+ *   h_init     optional fp32 [B, D] contiguous: h(-1).  NULL = zero.
+ *   h_final    optional fp32 [B, D] contiguous: receives h(L-1).  NULL = not wanted.
+ * All other arguments as qssm_scan_forward, which is this call with both set to NULL.
+ * No counterpart in the reference, whose recurrence always starts from h(-1) = 0
+ * (quick_ssm/scan_interface.py:15-21); its README lists a generation mode as future work
+ * (README.md:176-184).
+ */
+QSSM_API int qssm_scan_forward_carry(const qssm_plan* plan,
+                            const void* x, qssm_strides sx,
+                            const void* a, qssm_strides sa,
+                            const void* b, qssm_strides sb,
+                            const void* c, qssm_strides sc,
+                            void* y, qssm_strides sy,
+                            float* h_out, qssm_strides sh,
+                            float* ckpt,
+                            const float* h_init, float* h_final,
+                            void* control, uint64_t control_size,
+                            void* workspace, uint64_t workspace_bytes, uint32_t epoch,
+                            void* stream);
+
+/*
  * Backward scan: one reverse-time pass that reads x, a, b, c, dy once and writes dx, da, db,
  * dc once.  h is rebuilt inside each tile from `ckpt` (the checkpoint=True case), or read from
  * `h` when that is given (the checkpoint=False case and block_scan_backward_3d's signature);
@@ -188,6 +212,32 @@ QSSM_API int qssm_scan_backward(const qssm_plan* plan,
                        void* control, uint64_t control_size,
                        void* workspace, uint64_t workspace_bytes, uint32_t epoch,
                        void* stream);
+
+/*
+ * Backward scan with a carried state: the mirror image of qssm_scan_forward_carry.
+ *   h_init     the h(-1) the forward started from (needed for da at t = 0).  NULL = zero.
+ *   dh_final   optional fp32 [B, D]: gradient arriving at h(L-1) from whatever consumed h_final
+ *              (the next piece's dh_init when a sequence is scanned in pieces).  NULL = zero.
+ *   dh_init    optional fp32 [B, D]: receives the gradient of h(-1), a(0) * dH(0).  NULL = not wanted.
+ * All other arguments as qssm_scan_backward, which is this call with the three set to NULL.
+ * No counterpart in the reference (see qssm_scan_forward_carry).
+ */
+QSSM_API int qssm_scan_backward_carry(const qssm_plan* plan,
+                             const void* x, qssm_strides sx,
+                             const void* a, qssm_strides sa,
+                             const void* b, qssm_strides sb,
+                             const void* c, qssm_strides sc,
+                             const void* dy, qssm_strides sdy,
+                             const float* h, qssm_strides sh,
+                             const float* ckpt,
+                             const float* h_init, const float* dh_final, float* dh_init,
+                             void* dx, qssm_strides sdx,
+                             void* da, qssm_strides sda,
+                             void* db, qssm_strides sdb,
+                             void* dc, qssm_strides sdc,
+                             void* control, uint64_t control_size,
+                             void* workspace, uint64_t workspace_bytes, uint32_t epoch,
+                             void* stream);
 
 /*
  * Streaming copy of `bytes` bytes (16-byte aligned, multiple of 16) on `stream`.  Not part of

@@ -47,9 +47,12 @@ def _load() -> ctypes.CDLL:
         i = ctypes.c_int
         lib.oracle_scan_forward_f64.argtypes = [fp, fp, fp, fp, dp, dp, i, i, i]
         lib.oracle_scan_backward_f64.argtypes = [fp, fp, fp, fp, fp, dp, dp, dp, dp, i, i, i]
+        lib.oracle_scan_forward_carry_f64.argtypes = [fp, fp, fp, fp, fp, dp, dp, dp, i, i, i]
+        lib.oracle_scan_backward_carry_f64.argtypes = [fp] * 7 + [dp] * 5 + [i, i, i]
         lib.oracle_scan_forward_f32_seq.argtypes = [fp, fp, fp, fp, i, i, i]
         lib.oracle_scan_backward_f32_seq.argtypes = [fp] * 6 + [fp] * 4 + [i, i, i]
         for fn in (lib.oracle_scan_forward_f64, lib.oracle_scan_backward_f64,
+                   lib.oracle_scan_forward_carry_f64, lib.oracle_scan_backward_carry_f64,
                    lib.oracle_scan_forward_f32_seq, lib.oracle_scan_backward_f32_seq):
             fn.restype = None
         _lib = lib
@@ -92,6 +95,33 @@ def backward_f64(x, a, b, c, dy) -> Tuple[np.ndarray, np.ndarray, np.ndarray, np
     outs = [np.empty((B, L, D), dtype=np.float64) for _ in range(4)]
     _load().oracle_scan_backward_f64(_fp(x), _fp(a), _fp(b), _fp(c), _fp(dy), *[_dp(o) for o in outs], B, L, D)
     return tuple(outs)
+
+
+def forward_carry_f64(x, a, b, c, h0=None) -> Tuple[np.ndarray, np.ndarray, np.ndarray]:
+    """(h, y, h_final) in float64, the recurrence started from h(-1) = h0 ([B, D], None = zero)."""
+    x, a, b, c = (_f32(t) for t in (x, a, b, c))
+    B, L, D = x.shape
+    h0f = _f32(h0) if h0 is not None else None
+    h = np.empty((B, L, D), dtype=np.float64)
+    y = np.empty((B, L, D), dtype=np.float64)
+    hf = np.empty((B, D), dtype=np.float64)
+    _load().oracle_scan_forward_carry_f64(_fp(x), _fp(a), _fp(b), _fp(c), _fp(h0f) if h0f is not None else None,
+                                          _dp(h), _dp(y), _dp(hf), B, L, D)
+    return h, y, hf
+
+
+def backward_carry_f64(x, a, b, c, dy, h0=None, g_final=None):
+    """(dx, da, db, dc, dh0) in float64 for the loss sum(y * dy) + sum(h_final * g_final)."""
+    x, a, b, c, dy = (_f32(t) for t in (x, a, b, c, dy))
+    B, L, D = x.shape
+    h0f = _f32(h0) if h0 is not None else None
+    gf = _f32(g_final) if g_final is not None else None
+    outs = [np.empty((B, L, D), dtype=np.float64) for _ in range(4)]
+    dh0 = np.empty((B, D), dtype=np.float64)
+    _load().oracle_scan_backward_carry_f64(
+        _fp(x), _fp(a), _fp(b), _fp(c), _fp(dy), _fp(h0f) if h0f is not None else None,
+        _fp(gf) if gf is not None else None, *[_dp(o) for o in outs], _dp(dh0), B, L, D)
+    return tuple(outs) + (dh0,)
 
 
 def forward_f32_seq(x, a, b) -> np.ndarray:

@@ -26,8 +26,13 @@
 
 #define COLS 64 /* columns advanced together, for cache-friendly row access */
 
-void oracle_scan_forward_f64(const float* x, const float* a, const float* b, const float* c, double* h,
-                             double* y, int B, int L, int D) {
+/* The same recurrence started from h(-1) = h0[b, d] instead of zero (h0 may be NULL), also reporting
+ * h(L-1) in hfinal (may be NULL): what scanning a sequence in pieces hands from piece to piece.  The
+ * reference has no such entry (its h(-1) is always zero, quick_ssm/scan_interface.py:15-21); the
+ * recurrence itself is the one above.  Pinned by tests/test_oracle.py through the property that
+ * pieces chained this way reproduce the whole-sequence results of the functions below. */
+void oracle_scan_forward_carry_f64(const float* x, const float* a, const float* b, const float* c,
+                                   const float* h0, double* h, double* y, double* hfinal, int B, int L, int D) {
   const int nblk = (D + COLS - 1) / COLS;
 #pragma omp parallel for collapse(2) schedule(static)
   for (int bi = 0; bi < B; ++bi) {
@@ -35,6 +40,7 @@ void oracle_scan_forward_f64(const float* x, const float* a, const float* b, con
       const int d0 = blk * COLS, d1 = d0 + COLS < D ? d0 + COLS : D;
       double state[COLS];
       for (int k = 0; k < COLS; ++k) state[k] = 0.0;
+      if (h0) for (int d = d0; d < d1; ++d) state[d - d0] = (double)h0[(size_t)bi * D + d];
       for (int t = 0; t < L; ++t) {
         const size_t row = ((size_t)bi * L + t) * D;
         for (int d = d0; d < d1; ++d) {
@@ -44,13 +50,23 @@ void oracle_scan_forward_f64(const float* x, const float* a, const float* b, con
           if (y) y[row + d] = (c ? (double)c[row + d] : 1.0) * s;
         }
       }
+      if (hfinal) for (int d = d0; d < d1; ++d) hfinal[(size_t)bi * D + d] = state[d - d0];
     }
   }
 }
 
+void oracle_scan_forward_f64(const float* x, const float* a, const float* b, const float* c, double* h,
+                             double* y, int B, int L, int D) {
+  oracle_scan_forward_carry_f64(x, a, b, c, NULL, h, y, NULL, B, L, D);
+}
+
 /* h is rebuilt in double inside; hbuf holds one block of columns over all L. */
-void oracle_scan_backward_f64(const float* x, const float* a, const float* b, const float* c, const float* dy,
-                              double* dx, double* da, double* db, double* dc, int B, int L, int D) {
+/* Backward of the carried-state forward: g_final[b, d] (may be NULL) is the gradient arriving at h(L-1)
+ * from outside, so dh_next starts from it instead of zero; h(-1) = h0 enters da at t = 0; dh0 (may be
+ * NULL) receives the gradient of h0, which is dh_next after the last (t = 0) step. */
+void oracle_scan_backward_carry_f64(const float* x, const float* a, const float* b, const float* c, const float* dy,
+                                    const float* h0, const float* g_final, double* dx, double* da, double* db,
+                                    double* dc, double* dh0, int B, int L, int D) {
   const int nblk = (D + COLS - 1) / COLS;
 #pragma omp parallel for collapse(2) schedule(static)
   for (int bi = 0; bi < B; ++bi) {
@@ -59,6 +75,10 @@ void oracle_scan_backward_f64(const float* x, const float* a, const float* b, co
       double* hbuf = (double*)malloc((size_t)(L > 0 ? L : 1) * COLS * sizeof(double));
       double state[COLS], next[COLS];
       for (int k = 0; k < COLS; ++k) { state[k] = 0.0; next[k] = 0.0; }
+      for (int d = d0; d < d1; ++d) {
+        if (h0) state[d - d0] = (double)h0[(size_t)bi * D + d];
+        if (g_final) next[d - d0] = (double)g_final[(size_t)bi * D + d];
+      }
       for (int t = 0; t < L; ++t) {
         const size_t row = ((size_t)bi * L + t) * D;
         for (int d = d0; d < d1; ++d) {
@@ -71,7 +91,7 @@ void oracle_scan_backward_f64(const float* x, const float* a, const float* b, co
         for (int d = d0; d < d1; ++d) {
           const int k = d - d0;
           const double total = (double)dy[row + d] * (double)c[row + d] + next[k];
-          const double hprev = t > 0 ? hbuf[(size_t)(t - 1) * COLS + k] : 0.0;
+          const double hprev = t > 0 ? hbuf[(size_t)(t - 1) * COLS + k] : (h0 ? (double)h0[(size_t)bi * D + d] : 0.0);
           dc[row + d] = (double)dy[row + d] * hbuf[(size_t)t * COLS + k];
           db[row + d] = total * (double)x[row + d];
           da[row + d] = total * hprev;
@@ -79,9 +99,15 @@ void oracle_scan_backward_f64(const float* x, const float* a, const float* b, co
           next[k] = total * (double)a[row + d];
         }
       }
+      if (dh0) for (int d = d0; d < d1; ++d) dh0[(size_t)bi * D + d] = next[d - d0];
       free(hbuf);
     }
   }
+}
+
+void oracle_scan_backward_f64(const float* x, const float* a, const float* b, const float* c, const float* dy,
+                              double* dx, double* da, double* db, double* dc, int B, int L, int D) {
+  oracle_scan_backward_carry_f64(x, a, b, c, dy, NULL, NULL, dx, da, db, dc, NULL, B, L, D);
 }
 
 void oracle_scan_forward_f32_seq(const float* x, const float* a, const float* b, float* h, int B, int L, int D) {

@@ -6,6 +6,7 @@ from quick_ssm_amd.scan_interface import (  # noqa: F401
     _torch_scan,
     honor_tiles,
     scan,
+    scan_chunk,
 )
 
 __all__ = ["scan"]

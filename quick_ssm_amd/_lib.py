@@ -26,6 +26,8 @@ EXPORTED_SYMBOLS = (
     "qssm_control_status",
     "qssm_scan_forward",
     "qssm_scan_backward",
+    "qssm_scan_forward_carry",
+    "qssm_scan_backward_carry",
     "qssm_copy_bytes",
 )
 
@@ -98,6 +100,15 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.qssm_scan_backward.restype = ctypes.c_int
     lib.qssm_scan_backward.argtypes = (
         [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, Strides] * 4 + [vp, u64, vp, u64, ctypes.c_uint32, vp]
+    )
+    lib.qssm_scan_forward_carry.restype = ctypes.c_int
+    lib.qssm_scan_forward_carry.argtypes = (
+        [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, vp] + [vp, u64, vp, u64, ctypes.c_uint32, vp]
+    )
+    lib.qssm_scan_backward_carry.restype = ctypes.c_int
+    lib.qssm_scan_backward_carry.argtypes = (
+        [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, vp, vp] + [vp, Strides] * 4
+        + [vp, u64, vp, u64, ctypes.c_uint32, vp]
     )
     lib.qssm_copy_bytes.restype = ctypes.c_int
     lib.qssm_copy_bytes.argtypes = [vp, vp, u64, vp]

@@ -324,17 +324,28 @@ int qssm_scan_forward(const qssm_plan* plan, const void* x, qssm_strides sx, con
                       const void* b, qssm_strides sb, const void* c, qssm_strides sc, void* y, qssm_strides sy,
                       float* h_out, qssm_strides sh, float* ckpt, void* control, uint64_t control_size,
                       void* workspace, uint64_t workspace_bytes, uint32_t epoch, void* stream) {
+  return qssm_scan_forward_carry(plan, x, sx, a, sa, b, sb, c, sc, y, sy, h_out, sh, ckpt, nullptr, nullptr, control,
+                                 control_size, workspace, workspace_bytes, epoch, stream);
+}
+
+int qssm_scan_forward_carry(const qssm_plan* plan, const void* x, qssm_strides sx, const void* a, qssm_strides sa,
+                            const void* b, qssm_strides sb, const void* c, qssm_strides sc, void* y, qssm_strides sy,
+                            float* h_out, qssm_strides sh, float* ckpt, const float* h_init, float* h_final,
+                            void* control, uint64_t control_size, void* workspace, uint64_t workspace_bytes,
+                            uint32_t epoch, void* stream) {
   int rc = check_plan(plan, QSSM_FORWARD);
   if (rc != 0) return rc;
   if (plan->B == 0 || plan->L == 0 || plan->D == 0) return 0;
   if (x == nullptr || a == nullptr || b == nullptr) return fail(QSSM_EINVAL, "x, a, b must not be NULL");
-  if (y == nullptr && h_out == nullptr && ckpt == nullptr) return fail(QSSM_EINVAL, "no output requested");
+  if (y == nullptr && h_out == nullptr && ckpt == nullptr && h_final == nullptr)
+    return fail(QSSM_EINVAL, "no output requested");
   fwd_launch_fn fn = find_fwd_launcher(plan->in_dtype, plan->out_dtype);
   if (fn == nullptr) return fail(QSSM_EINVAL, "dtype pair is not built");
   const int es = dtype_size(plan->in_dtype), os = dtype_size(plan->out_dtype), v = plan->vec;
   if (!aligned_to(x, sx.b, sx.l, es, v) || !aligned_to(a, sa.b, sa.l, es, v) || !aligned_to(b, sb.b, sb.l, es, v) ||
       !aligned_to(c, sc.b, sc.l, es, v) || !aligned_to(y, sy.b, sy.l, os, v) ||
-      !aligned_to(h_out, sh.b, sh.l, 4, v) || !aligned_to(ckpt, 0, 0, 4, v))
+      !aligned_to(h_out, sh.b, sh.l, 4, v) || !aligned_to(ckpt, 0, 0, 4, v) || !aligned_to(h_init, 0, 0, 4, v) ||
+      !aligned_to(h_final, 0, 0, 4, v))
     return fail(QSSM_EALIGN, "a pointer or stride is not aligned to plan.vec=%d elements", v);
   if (control == nullptr || control_size < plan->control_bytes)
     return fail(QSSM_EWORKSPACE, "control block has %llu bytes, plan needs %llu", (unsigned long long)control_size,
@@ -354,6 +365,7 @@ int qssm_scan_forward(const qssm_plan* plan, const void* x, qssm_strides sx, con
   FwdArgs args;
   fill_geometry(&args.g, plan, control, workspace, epoch);
   args.x = x; args.a = a; args.b = b; args.c = c; args.y = y; args.h_out = h_out; args.ckpt = ckpt;
+  args.h_init = h_init; args.h_final = h_final;
   args.x_sb = sx.b; args.x_sl = sx.l; args.a_sb = sa.b; args.a_sl = sa.l;
   args.b_sb = sb.b; args.b_sl = sb.l; args.c_sb = sc.b; args.c_sl = sc.l;
   args.y_sb = sy.b; args.y_sl = sy.l; args.h_sb = sh.b; args.h_sl = sh.l;
@@ -378,6 +390,18 @@ int qssm_scan_backward(const qssm_plan* plan, const void* x, qssm_strides sx, co
                        qssm_strides sdx, void* da, qssm_strides sda, void* db, qssm_strides sdb, void* dc,
                        qssm_strides sdc, void* control, uint64_t control_size, void* workspace,
                        uint64_t workspace_bytes, uint32_t epoch, void* stream) {
+  return qssm_scan_backward_carry(plan, x, sx, a, sa, b, sb, c, sc, dy, sdy, h, sh, ckpt, nullptr, nullptr, nullptr, dx,
+                                  sdx, da, sda, db, sdb, dc, sdc, control, control_size, workspace, workspace_bytes,
+                                  epoch, stream);
+}
+
+int qssm_scan_backward_carry(const qssm_plan* plan, const void* x, qssm_strides sx, const void* a, qssm_strides sa,
+                             const void* b, qssm_strides sb, const void* c, qssm_strides sc, const void* dy,
+                             qssm_strides sdy, const float* h, qssm_strides sh, const float* ckpt,
+                             const float* h_init, const float* dh_final, float* dh_init, void* dx, qssm_strides sdx,
+                             void* da, qssm_strides sda, void* db, qssm_strides sdb, void* dc, qssm_strides sdc,
+                             void* control, uint64_t control_size, void* workspace, uint64_t workspace_bytes,
+                             uint32_t epoch, void* stream) {
   int rc = check_plan(plan, QSSM_BACKWARD);
   if (rc != 0) return rc;
   if (plan->B == 0 || plan->L == 0 || plan->D == 0) return 0;
@@ -389,7 +413,8 @@ int qssm_scan_backward(const qssm_plan* plan, const void* x, qssm_strides sx, co
   const int es = dtype_size(plan->in_dtype), os = dtype_size(plan->out_dtype), v = plan->vec;
   if (!aligned_to(x, sx.b, sx.l, es, v) || !aligned_to(a, sa.b, sa.l, es, v) || !aligned_to(b, sb.b, sb.l, es, v) ||
       !aligned_to(c, sc.b, sc.l, es, v) || !aligned_to(dy, sdy.b, sdy.l, os, v) ||
-      !aligned_to(h, sh.b, sh.l, 4, v) || !aligned_to(ckpt, 0, 0, 4, v) || !aligned_to(dx, sdx.b, sdx.l, es, v) ||
+      !aligned_to(h, sh.b, sh.l, 4, v) || !aligned_to(ckpt, 0, 0, 4, v) || !aligned_to(h_init, 0, 0, 4, v) ||
+      !aligned_to(dh_final, 0, 0, 4, v) || !aligned_to(dh_init, 0, 0, 4, v) || !aligned_to(dx, sdx.b, sdx.l, es, v) ||
       !aligned_to(da, sda.b, sda.l, es, v) || !aligned_to(db, sdb.b, sdb.l, es, v) ||
       !aligned_to(dc, sdc.b, sdc.l, es, v))
     return fail(QSSM_EALIGN, "a pointer or stride is not aligned to plan.vec=%d elements", v);
@@ -413,6 +438,7 @@ int qssm_scan_backward(const qssm_plan* plan, const void* x, qssm_strides sx, co
   BwdArgs args;
   fill_geometry(&args.g, plan, control, workspace, epoch);
   args.x = x; args.a = a; args.b = b; args.c = c; args.dy = dy; args.h = h; args.ckpt = ckpt;
+  args.h_init = h_init; args.dh_final = dh_final; args.dh_init = dh_init;
   args.dx = dx; args.da = da; args.db = db; args.dc = dc;
   args.x_sb = sx.b; args.x_sl = sx.l; args.a_sb = sa.b; args.a_sl = sa.l;
   args.b_sb = sb.b; args.b_sl = sb.l; args.c_sb = sc.b; args.c_sl = sc.l;

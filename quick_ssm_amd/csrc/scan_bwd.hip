@@ -191,11 +191,20 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
       const Pack<float, VEC> hv = load_pack<float, VEC>(hp - p.h_sl);
 #pragma unroll
       for (int v = 0; v < VEC; ++v) hprev[v] = hv.v[v];
+    } else if (dok && t0 == 0 && p.h_init != nullptr) {
+      const Pack<float, VEC> hv = load_pack<float, VEC>(p.h_init + (int64_t)bi * g.D + d);
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) hprev[v] = hv.v[v];
     }
   } else if (dok && t_tile > 0) {
     // state at the tile's first step, saved by the forward
     const Pack<float, VEC> hv = load_pack<float, VEC>(
         p.ckpt + ((int64_t)bi * g.n_ckpt + t_tile / g.ckpt_stride) * g.D + d);
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) hprev[v] = hv.v[v];
+  } else if (dok && p.h_init != nullptr) {
+    // the first tile starts from the carried-in state
+    const Pack<float, VEC> hv = load_pack<float, VEC>(p.h_init + (int64_t)bi * g.D + d);
 #pragma unroll
     for (int v = 0; v < VEC; ++v) hprev[v] = hv.v[v];
   }
@@ -206,6 +215,13 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   float ein[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; ++v) ein[v] = 0.0f;
+  // A gradient arriving at the final state enters where the zero carry would: at the last cluster's
+  // tiles (the lane group that folds the neighbours' maps onto it), or at every lane of a lone tile.
+  if (p.dh_final != nullptr && s == g.n_super - 1 && dok && (edge || !multi)) {
+    const Pack<float, VEC> ev = load_pack<float, VEC>(p.dh_final + (int64_t)bi * g.D + d);
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) ein[v] = ev.v[v];
+  }
   if (want_state && pk_state.ready(g.epoch)) {
     state_here = true;
 #pragma unroll
@@ -412,6 +428,13 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
     }
     // Keep each step's conversions next to their use (register footprint).
     __builtin_amdgcn_sched_barrier(0);
+  }
+  // What leaves the first step backwards, a(0) * dH(0), is the gradient of the carried-in state.
+  if (p.dh_init != nullptr && seg == 0 && j == 0 && dok) {
+    Pack<float, VEC> ev;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) ev.v[v] = E[v];
+    store_pack<float, VEC>(p.dh_init + (int64_t)bi * g.D + d, ev);
   }
 }
 

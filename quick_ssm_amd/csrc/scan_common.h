@@ -375,6 +375,8 @@ struct FwdArgs {
   void* y;
   float* h_out;
   float* ckpt;
+  const float* h_init;  // [B, D] state before the first step (null: zero)
+  float* h_final;       // [B, D] state after the last step (null: not wanted)
   int64_t x_sb, x_sl, a_sb, a_sl, b_sb, b_sl, c_sb, c_sl, y_sb, y_sl, h_sb, h_sl;
 };
 
@@ -383,6 +385,9 @@ struct BwdArgs {
   const void *x, *a, *b, *c, *dy;
   const float* h;
   const float* ckpt;
+  const float* h_init;    // [B, D] state before the first step (null: zero)
+  const float* dh_final;  // [B, D] gradient arriving at the state after the last step (null: zero)
+  float* dh_init;         // [B, D] gradient of the state before the first step (null: not wanted)
   void *dx, *da, *db, *dc;
   int64_t x_sb, x_sl, a_sb, a_sl, b_sb, b_sl, c_sb, c_sl, dy_sb, dy_sl, h_sb, h_sl;
   int64_t dx_sb, dx_sl, da_sb, da_sl, db_sb, db_sl, dc_sb, dc_sl;

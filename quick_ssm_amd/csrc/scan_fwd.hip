@@ -150,6 +150,13 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   float hin[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; ++v) hin[v] = 0.0f;
+  // A carried-in state enters where the zero state would: at the first cluster's tiles (the lane group
+  // that folds the neighbours' maps onto it), or at every lane when the chain has a single tile.
+  if (p.h_init != nullptr && s == 0 && dok && (edge || !multi)) {
+    const Pack<float, VEC> hv = load_pack<float, VEC>(p.h_init + (int64_t)bi * g.D + d);
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) hin[v] = hv.v[v];
+  }
   if (want_map && pk_map.ready(g.epoch)) {
     map_here = true;
     float wa[VEC], wx[VEC];
@@ -293,7 +300,8 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
     for (int v = 0; v < VEC; ++v) hv.v[v] = h[v];
     store_pack<float, VEC>(p.ckpt + ((int64_t)bi * g.n_ckpt + t0 / g.ckpt_stride) * g.D + d, hv);
   }
-  if (!want_y && p.h_out == nullptr) return;
+  const bool want_final = p.h_final != nullptr && seg == g.n_seg - 1 && edge;
+  if (!want_y && p.h_out == nullptr && p.h_final == nullptr) return;
 
   // ---- sweep 2: the recurrence proper, from the true carry-in -----------------------------------
   char* yb = (char*)p.y + ((int64_t)bi * p.y_sb + (int64_t)t_tile * p.y_sl + col0) * (int64_t)sizeof(Tout);
@@ -318,6 +326,13 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
     // Keep each step's conversions next to their use: hoisting them all above the recurrence
     // would hold an fp32 copy of the whole tile in registers.
     __builtin_amdgcn_sched_barrier(0);
+  }
+  // Steps past L are identity steps, so the last lane group of the last tile ends on h(L-1).
+  if (want_final && dok) {
+    Pack<float, VEC> hv;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) hv.v[v] = h[v];
+    store_pack<float, VEC>(p.h_final + (int64_t)bi * g.D + d, hv);
   }
 }
 

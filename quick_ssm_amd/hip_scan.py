@@ -158,6 +158,15 @@ def _require_gpu(*tensors: Tensor) -> torch.device:
     return dev
 
 
+def _check_state(t: Optional[Tensor], B: int, D: int, dev: torch.device, name: str) -> None:
+    """A carried state / its gradient: fp32 [B, D], contiguous, on the operands' device."""
+    if t is None:
+        return
+    if tuple(t.shape) != (B, D) or t.dtype != torch.float32 or not t.is_contiguous() or t.device != dev:
+        raise ValueError(f"{name} must be a contiguous float32 tensor of shape {(B, D)} on {dev}, "
+                         f"got {t.dtype} {tuple(t.shape)} on {t.device}")
+
+
 def scan_forward(
     x: Tensor, a: Tensor, b: Tensor, c: Optional[Tensor], *,
     out_dtype: torch.dtype,
@@ -166,12 +175,15 @@ def scan_forward(
     want_ckpt: bool = True,
     tune: int = 0,
     bwd_tune: int = 0,
+    h_init: Optional[Tensor] = None,
+    h_final: Optional[Tensor] = None,
 ) -> Tuple[Optional[Tensor], Optional[Tensor], Optional[Tensor], int]:
     """One forward launch.  Operands must already share one supported storage type.
 
     Returns (y, h, ckpt, ckpt_stride): y in `out_dtype` (a storage the kernels are built for), h
     the full fp32 state if `want_h`, ckpt the fp32 states h(t-1) at t = k*ckpt_stride if
-    `want_ckpt` (what the backward rebuilds h from).
+    `want_ckpt` (what the backward rebuilds h from).  `h_init` (fp32 [B, D], contiguous) is the
+    state before the first step instead of zero; `h_final` (same layout) receives h(L-1).
     """
     ops = [x, a, b] + ([c] if c is not None else [])
     dev = _require_gpu(*ops)
@@ -179,7 +191,11 @@ def scan_forward(
     in_dtype = x.dtype
     y = torch.empty((B, L, D), dtype=out_dtype, device=dev) if want_y else None
     h = torch.empty((B, L, D), dtype=torch.float32, device=dev) if want_h else None
+    _check_state(h_init, B, D, dev, "h_init")
+    _check_state(h_final, B, D, dev, "h_final")
     if B == 0 or L == 0 or D == 0:
+        if h_final is not None:  # nothing happened to the state
+            h_final.copy_(h_init) if h_init is not None else h_final.zero_()
         return y, h, (torch.empty((B, 0, D), dtype=torch.float32, device=dev) if want_ckpt else None), 0
 
     x, a, b = _unit_inner(x), _unit_inner(a), _unit_inner(b)
@@ -199,10 +215,10 @@ def scan_forward(
         stream = torch.cuda.current_stream(dev).cuda_stream
         ctl, ws, epoch = _launch_buffers(dev, stream, plan)
         _lib.check(
-            _lib.load().qssm_scan_forward(
+            _lib.load().qssm_scan_forward_carry(
                 ctypes.byref(plan),
                 _ptr(x), _strides(x), _ptr(a), _strides(a), _ptr(b), _strides(b), _ptr(c), _strides(c),
-                _ptr(y), _strides(y), _ptr(h), _strides(h), _ptr(ckpt),
+                _ptr(y), _strides(y), _ptr(h), _strides(h), _ptr(ckpt), _ptr(h_init), _ptr(h_final),
                 ctl.data_ptr(), ctl.numel(), ws.data_ptr(), ws.numel(), epoch, stream,
             )
         )
@@ -216,17 +232,26 @@ def scan_backward(
     ckpt_stride: int = 0,
     need: Sequence[bool] = (True, True, True, True),
     tune: int = 0,
+    h_init: Optional[Tensor] = None,
+    dh_final: Optional[Tensor] = None,
+    dh_init: Optional[Tensor] = None,
 ) -> Tuple[Optional[Tensor], Optional[Tensor], Optional[Tensor], Optional[Tensor]]:
     """One backward launch.  x, a, b, c share one storage type; dy has the storage of y.
 
     Exactly one of `h` (full fp32 state) and `ckpt` (+ its `ckpt_stride`) must be given.  Returns
     (dx, da, db, dc) in the storage type of the operands; entries not in `need` are None.
+    `h_init` is the state the forward started from, `dh_final` the gradient arriving at h(L-1),
+    `dh_init` receives the gradient of h(-1); all fp32 [B, D], contiguous, optional.
     """
     dev = _require_gpu(x, a, b, c, dy)
     B, L, D = x.shape
     in_dtype = x.dtype
     grads = [torch.empty((B, L, D), dtype=in_dtype, device=dev) if n else None for n in need]
+    for name, t in (("h_init", h_init), ("dh_final", dh_final), ("dh_init", dh_init)):
+        _check_state(t, B, D, dev, name)
     if B == 0 or L == 0 or D == 0:
+        if dh_init is not None:  # the state passed through untouched
+            dh_init.copy_(dh_final) if dh_final is not None else dh_init.zero_()
         return tuple(grads)
     if (h is None) == (ckpt is None):
         raise ValueError("pass exactly one of h and ckpt")
@@ -245,10 +270,11 @@ def scan_backward(
         stream = torch.cuda.current_stream(dev).cuda_stream
         ctl, ws, epoch = _launch_buffers(dev, stream, plan)
         _lib.check(
-            _lib.load().qssm_scan_backward(
+            _lib.load().qssm_scan_backward_carry(
                 ctypes.byref(plan),
                 _ptr(x), _strides(x), _ptr(a), _strides(a), _ptr(b), _strides(b), _ptr(c), _strides(c),
                 _ptr(dy), _strides(dy), _ptr(h), _strides(h), _ptr(ckpt),
+                _ptr(h_init), _ptr(dh_final), _ptr(dh_init),
                 _ptr(grads[0]), _strides(grads[0]), _ptr(grads[1]), _strides(grads[1]),
                 _ptr(grads[2]), _strides(grads[2]), _ptr(grads[3]), _strides(grads[3]),
                 ctl.data_ptr(), ctl.numel(), ws.data_ptr(), ws.numel(), epoch, stream,

@@ -9,7 +9,7 @@ every element still sees the same operations in the same order.
 """
 from __future__ import annotations
 
-from typing import Tuple
+from typing import Optional, Tuple
 
 import torch
 
@@ -18,19 +18,26 @@ Tensor = torch.Tensor
 _HALF = (torch.float16, torch.bfloat16)
 
 
-def naive_forward_3d(x: Tensor, a: Tensor, b: Tensor) -> Tensor:
-    """h(t) = a(t) * h(t-1) + b(t) * x(t) with h(-1) = 0, for [B, L, D] tensors; returns h in x.dtype."""
+def naive_forward_3d(x: Tensor, a: Tensor, b: Tensor, h_init: Optional[Tensor] = None,
+                     return_final: bool = False):
+    """h(t) = a(t) * h(t-1) + b(t) * x(t) for [B, L, D] tensors; returns h in x.dtype.
+
+    h(-1) is zero, as in the reference, unless `h_init` ([B, D]) is given.  With `return_final` the
+    state after the last step comes back too, in the accumulation dtype: (h, h_final).
+    """
     B, L, D = x.shape
     acc = torch.float32 if x.dtype in _HALF else x.dtype
     xs, as_, bs = x.to(acc), a.to(acc), b.to(acc)
-    if L == 0:
-        return torch.zeros((B, L, D), device=x.device, dtype=x.dtype)
-    state = torch.zeros((B, D), device=x.device, dtype=acc)
+    if h_init is None:
+        state = torch.zeros((B, D), device=x.device, dtype=acc)
+    else:
+        state = h_init.to(acc)
     steps = []
     for t in range(L):
         state = as_[:, t] * state + bs[:, t] * xs[:, t]
         steps.append(state)
-    return torch.stack(steps, dim=1).to(x.dtype)
+    h = torch.stack(steps, dim=1).to(x.dtype) if L > 0 else torch.zeros((B, L, D), device=x.device, dtype=x.dtype)
+    return (h, state) if return_final else h
 
 
 def naive_full_3d(x: Tensor, a: Tensor, b: Tensor, c: Tensor) -> Tuple[Tensor, Tensor]:

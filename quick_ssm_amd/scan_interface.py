@@ -161,6 +161,109 @@ def _torch_scan(x: Tensor, a: Tensor, b: Tensor, c: Tensor, out_dtype: torch.dty
     return (c * h).to(out_dtype)
 
 
+class _HipScanCarryFunction(torch.autograd.Function):
+    """Autograd node of the device scan with a carried state: (x, a, b, c, h_init) -> (y, h_final).
+
+    One HIP launch forward, one backward, like `_HipScanFunction`; the backward also takes the
+    gradient arriving at h_final and returns the gradient of h_init, so pieces of a sequence
+    chain through autograd exactly as the whole sequence would.
+    """
+
+    @staticmethod
+    def forward(ctx, x: Tensor, a: Tensor, b: Tensor, c: Tensor, h_init: Optional[Tensor], checkpoint: bool,
+                out_dtype: torch.dtype):
+        if x.shape != a.shape or x.shape != b.shape or x.shape != c.shape:
+            raise ValueError("x, a, b, c must share the same shape [B, L, D].")
+        if x.dim() != 3:
+            raise ValueError("x, a, b, c must be 3-D tensors [B, L, D].")
+        if x.device.type != "cuda":
+            raise RuntimeError("HIP scan backend requires GPU tensors.")
+        B, L, D = x.shape
+        if h_init is not None and tuple(h_init.shape) != (B, D):
+            raise ValueError(f"state must have shape {(B, D)}, got {tuple(h_init.shape)}.")
+        k_in, k_out = hip_scan.kernel_dtypes([x.dtype, a.dtype, b.dtype, c.dtype], out_dtype)
+        xs, as_, bs, cs = (t if t.dtype == k_in else t.to(k_in) for t in (x, a, b, c))
+        h0 = None
+        if h_init is not None:
+            h0 = h_init.detach().to(torch.float32).contiguous()
+            if h0.data_ptr() % 16 != 0:
+                h0 = h0.clone()
+        h_final = torch.empty((B, D), dtype=torch.float32, device=x.device)
+        y, h_full, ckpt, stride = hip_scan.scan_forward(
+            xs, as_, bs, cs, out_dtype=k_out, want_h=not checkpoint, want_ckpt=bool(checkpoint),
+            h_init=h0, h_final=h_final,
+        )
+        ctx.save_for_backward(x, a, b, c)
+        ctx.k_in, ctx.k_out = k_in, k_out
+        ctx.h0, ctx.h_saved, ctx.ckpt, ctx.stride = h0, h_full, ckpt, stride
+        ctx.state_dtype = None if h_init is None else h_init.dtype
+        return (y if y.dtype == out_dtype else y.to(out_dtype)), h_final
+
+    @staticmethod
+    def backward(ctx, grad_y: Optional[Tensor], grad_state: Optional[Tensor]):
+        x, a, b, c = ctx.saved_tensors
+        k_in, k_out = ctx.k_in, ctx.k_out
+        B, L, D = x.shape
+        xs, as_, bs, cs = (t if t.dtype == k_in else t.to(k_in) for t in (x, a, b, c))
+        if grad_y is None:
+            grad_y = torch.zeros((B, L, D), dtype=k_out, device=x.device)
+        dy = grad_y if grad_y.dtype == k_out else grad_y.to(k_out)
+        dh_final = None
+        if grad_state is not None:
+            dh_final = grad_state.to(torch.float32).contiguous()
+            if dh_final.data_ptr() % 16 != 0:
+                dh_final = dh_final.clone()
+        need = tuple(ctx.needs_input_grad[:4])
+        dh_init = None
+        if ctx.needs_input_grad[4]:
+            dh_init = torch.empty((B, D), dtype=torch.float32, device=x.device)
+        out = hip_scan.scan_backward(
+            xs, as_, bs, cs, dy, h=ctx.h_saved, ckpt=None if ctx.h_saved is not None else ctx.ckpt,
+            ckpt_stride=ctx.stride, need=need, h_init=ctx.h0, dh_final=dh_final, dh_init=dh_init,
+        )
+
+        def _as(g: Optional[Tensor], like_dtype) -> Optional[Tensor]:
+            if g is None:
+                return None
+            return g if g.dtype == like_dtype else g.to(like_dtype)
+
+        return (_as(out[0], x.dtype), _as(out[1], a.dtype), _as(out[2], b.dtype), _as(out[3], c.dtype),
+                _as(dh_init, ctx.state_dtype), None, None)
+
+
+def scan_chunk(
+    x: Tensor,
+    a: Tensor,
+    b: Tensor,
+    c: Tensor,
+    state: Optional[Tensor] = None,
+    *,
+    checkpoint: bool = True,
+    backend: str = "auto",
+    out_dtype: Optional[torch.dtype] = None,
+) -> Tuple[Tensor, Tensor]:
+    """One piece of a longer scan: starts from `state` (h before the piece's first step, [B, D]; None
+    = zero) and returns `(y, new_state)` with new_state = h after its last step, in float32 (on the
+    sequential CPU path: in the dtype the recurrence is accumulated in).
+
+    Feeding each piece's `new_state` to the next gives the same y, and through autograd the same
+    gradients, as one `scan` over the concatenated sequence: chunked prefill and token-by-token
+    generation (L = 1).  The reference's scan always starts from zero
+    (quick_ssm/scan_interface.py:15-21) and lists a generation mode as future work (README.md:176-184);
+    this is that mode on the same kernels.
+    """
+    out_dtype = out_dtype or x.dtype
+    chosen = backend
+    if backend == "auto":
+        chosen = "hip" if x.device.type == "cuda" else "torch"
+    if chosen in ("hip", "triton"):
+        return _HipScanCarryFunction.apply(x, a, b, c, state, checkpoint, out_dtype)
+    if chosen == "torch":
+        h, final = naive_forward_3d(x, a, b, h_init=state, return_final=True)
+        return (c * h).to(out_dtype), final
+    raise ValueError(f"Unsupported backend '{backend}'. Use 'auto', 'hip', 'triton', or 'torch'.")
+
+
 def scan(
     x: Tensor,
     a: Tensor,
@@ -196,4 +299,4 @@ def scan(
     raise ValueError(f"Unsupported backend '{backend}'. Use 'auto', 'hip', 'triton', or 'torch'.")
 
 
-__all__ = ["scan", "honor_tiles"]
+__all__ = ["scan", "scan_chunk", "honor_tiles"]

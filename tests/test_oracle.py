@@ -122,6 +122,61 @@ def test_time_concatenation_property():
     np.testing.assert_allclose(np.stack(tail, axis=1), h_full[:, k:], rtol=1e-13)
 
 
+def test_carried_state_pieces_reproduce_the_whole_sequence():
+    # Pins the carried-state oracle functions on the whole-sequence ones (which the exact vectors, closed forms and
+    # finite differences above pin): scanning [0, L) in pieces, handing h_final on as the next piece's h0, must give
+    # the same h and y; and running the pieces' backward passes last piece first, handing dh0 back as the previous
+    # piece's incoming gradient of h_final, must give the same gradients.  The carried values are float32 (what the
+    # device hands over), so agreement is to float32 rounding of the state, not to float64.
+    x, a, b, c, dy = make_inputs((2, 61, 5), seed=23)
+    h_full, y_full = oracle.forward_f64(x, a, b, c)
+    g_full = oracle.backward_f64(x, a, b, c, dy)
+    cuts = [0, 1, 18, 19, 40, 61]
+    pieces = list(zip(cuts[:-1], cuts[1:]))
+    h0, states, hs, ys = None, [], [], []
+    for k0, k1 in pieces:
+        states.append(h0)
+        h, y, hf = oracle.forward_carry_f64(x[:, k0:k1], a[:, k0:k1], b[:, k0:k1], c[:, k0:k1], h0)
+        np.testing.assert_array_equal(hf, h[:, -1])
+        hs.append(h)
+        ys.append(y)
+        h0 = hf.astype(np.float32)
+    np.testing.assert_allclose(np.concatenate(hs, 1), h_full, rtol=0, atol=2e-7 * np.abs(h_full).max())
+    np.testing.assert_allclose(np.concatenate(ys, 1), y_full, rtol=0, atol=2e-7 * np.abs(y_full).max())
+    g_in, grads = None, []
+    for (k0, k1), st in reversed(list(zip(pieces, states))):
+        out = oracle.backward_carry_f64(x[:, k0:k1], a[:, k0:k1], b[:, k0:k1], c[:, k0:k1], dy[:, k0:k1], st, g_in)
+        grads.append(out[:4])
+        g_in = out[4].astype(np.float32)
+    grads.reverse()
+    for k in range(4):
+        got = np.concatenate([g[k] for g in grads], 1)
+        np.testing.assert_allclose(got, g_full[k], rtol=0, atol=1e-6 * np.abs(g_full[k]).max())
+
+
+def test_carried_state_gradients_by_finite_differences():
+    # d loss / d h0 and the effect of an incoming gradient on h_final, checked against central differences of
+    # loss(h0) = sum(y * dy) + sum(h_final * g_final), which is affine in h0 (so the difference is exact up to rounding).
+    x, a, b, c, dy = make_inputs((1, 9, 3), seed=29)
+    rng = np.random.default_rng(5)
+    h0 = rng.standard_normal((1, 3)).astype(np.float32)
+    g_final = rng.standard_normal((1, 3)).astype(np.float32)
+
+    def loss(h0v):
+        _, y, hf = oracle.forward_carry_f64(x, a, b, c, h0v)
+        return float((y * dy.double().numpy()).sum() + (hf * g_final).sum())
+
+    dh0 = oracle.backward_carry_f64(x, a, b, c, dy, h0, g_final)[4]
+    for d in range(3):
+        step = np.zeros_like(h0)
+        step[0, d] = 0.5
+        fd = (loss(h0 + step) - loss(h0 - step)) / float((h0 + step)[0, d] - (h0 - step)[0, d])
+        assert abs(fd - dh0[0, d]) <= 1e-6 * max(1.0, abs(fd))
+    # with L = 0 nothing touches the state: dh0 is the incoming gradient
+    e = np.zeros((1, 0, 3), dtype=np.float32)
+    np.testing.assert_array_equal(oracle.backward_carry_f64(e, e, e, e, e, h0, g_final)[4], g_final.astype(np.float64))
+
+
 def test_c_and_torch_flavours_agree_bitwise_in_fp32():
     x, a, b, c, dy = make_inputs((2, 130, 5), seed=3)
     h_c = oracle.forward_f32_seq(x, a, b)

@@ -14,7 +14,7 @@ import torch
 import oracle
 from helpers import TOL, assert_close, make_inputs, oracle_all, run_scan_with_grads
 from quick_ssm_amd import _lib, hip_scan
-from quick_ssm_amd.scan_interface import honor_tiles, scan
+from quick_ssm_amd.scan_interface import honor_tiles, scan, scan_chunk
 
 pytestmark = pytest.mark.gpu
 
@@ -224,6 +224,96 @@ def test_non_contiguous_operands(gpu):
     for k, t in zip(("dx", "da", "db", "dc"), leaves):
         got[k] = t.grad.cpu()
     _check_all(got, ref, 1e-5)
+
+
+# ---- carried state: a sequence scanned in pieces ------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype,shape,cuts", [
+    (torch.float32, (2, 777, 64), [0, 1, 300, 301, 777]),
+    (torch.bfloat16, (2, 1100, 264), [0, 5, 600, 1100]),
+    (torch.float16, (3, 40, 6), [0, 1, 2, 3, 40]),
+], ids=["f32", "bf16", "f16"])
+def test_pieces_with_carried_state_equal_the_whole_scan(gpu, dtype, shape, cuts):
+    x, a, b, c, dy = make_inputs(shape, dtype=dtype, seed=41)
+    ref = oracle_all(x, a, b, c, dy)
+    h64, _ = oracle.forward_f64(x, a, b, c)
+    leaves = [t.to(gpu).requires_grad_(True) for t in (x, a, b, c)]
+    state, ys = None, []
+    for k0, k1 in zip(cuts[:-1], cuts[1:]):
+        y, state = scan_chunk(*(t[:, k0:k1] for t in leaves), state)
+        assert state.dtype == torch.float32 and state.shape == (shape[0], shape[2])
+        assert_close(f"state after step {k1 - 1}", state.detach(), h64[:, k1 - 1], 1e-5)
+        ys.append(y)
+    y = torch.cat(ys, dim=1)
+    y.backward(dy.to(gpu))
+    got = {"y": y.detach().cpu()}
+    for k, t in zip(("dx", "da", "db", "dc"), leaves):
+        got[k] = t.grad.cpu()
+    _check_all(got, ref, TOL[dtype])
+    whole = run_scan_with_grads(scan, x, a, b, c, dy, gpu)
+    for k in got:  # and the one-launch scan says the same
+        assert_close(k + " (pieces vs whole)", got[k], whole[k].double().numpy(), TOL[dtype])
+
+
+def test_token_by_token_generation_matches_scan(gpu):
+    x, a, b, c, _ = make_inputs((2, 12, 520), dtype=torch.float16, seed=43)
+    dev = [t.to(gpu) for t in (x, a, b, c)]
+    whole = scan(*dev)
+    state, steps = None, []
+    with torch.no_grad():
+        for t in range(12):
+            y, state = scan_chunk(*(v[:, t:t + 1] for v in dev), state)
+            steps.append(y)
+    h64, y64 = oracle.forward_f64(x, a, b, c)
+    assert_close("y", torch.cat(steps, 1).cpu(), y64, TOL[torch.float16])
+    assert_close("y vs scan", torch.cat(steps, 1).cpu(), whole.double().cpu().numpy(), TOL[torch.float16])
+    assert_close("state", state.cpu(), h64[:, -1], 1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("keep_h", [False, True], ids=["ckpt", "full_h"])
+def test_carried_state_through_clustered_chains_and_its_gradients(gpu, dtype, keep_h):
+    # 64-lane rows, clusters of two: the state enters the first cluster's tiles, the incoming gradient the last
+    # cluster's, and both must come out right at the other end (oracle: the carried-state recurrence in float64).
+    shape = (2, 700, 512)
+    x, a, b, c, dy = make_inputs(shape, dtype=dtype, seed=47)
+    rng = np.random.default_rng(7)
+    h0 = torch.from_numpy(rng.standard_normal((shape[0], shape[2])).astype(np.float32))
+    g_final = torch.from_numpy(rng.standard_normal((shape[0], shape[2])).astype(np.float32))
+    _, y64, hf64 = oracle.forward_carry_f64(x, a, b, c, h0)
+    ref = oracle.backward_carry_f64(x, a, b, c, dy, h0, g_final)
+    tune = 7 | (8 << 8) | (2 << 28)
+    ops = [t.to(gpu) for t in (x, a, b, c)]
+    h_final = torch.empty(shape[0], shape[2], dtype=torch.float32, device=gpu)
+    dh_init = torch.empty_like(h_final)
+    y, h, ckpt, stride = hip_scan.scan_forward(*ops, out_dtype=dtype, want_h=keep_h, want_ckpt=not keep_h, tune=tune,
+                                               bwd_tune=tune, h_init=h0.to(gpu), h_final=h_final)
+    grads = hip_scan.scan_backward(*ops, dy.to(gpu), h=h, ckpt=ckpt, ckpt_stride=stride, tune=tune,
+                                   h_init=h0.to(gpu), dh_final=g_final.to(gpu), dh_init=dh_init)
+    assert hip_scan.workspace_status() == 0
+    assert_close("y", y.cpu(), y64, TOL[dtype])
+    assert_close("h_final", h_final.cpu(), hf64, 1e-5)
+    for name, got, want in zip(("dx", "da", "db", "dc"), grads, ref[:4]):
+        assert_close(name, got.cpu(), want, TOL[dtype])
+    assert_close("dh_init", dh_init.cpu(), ref[4], 1e-5)
+
+
+def test_carried_state_argument_errors_and_empty_piece(gpu):
+    x, a, b, c, _ = make_inputs((2, 8, 4), seed=3)
+    dev = [t.to(gpu) for t in (x, a, b, c)]
+    with pytest.raises(ValueError):
+        scan_chunk(*dev, torch.zeros(2, 5, device=gpu))
+    with pytest.raises(ValueError):
+        hip_scan.scan_forward(*dev, out_dtype=torch.float32, h_init=torch.zeros(2, 4, device=gpu, dtype=torch.float16))
+    st = torch.arange(8, dtype=torch.float32, device=gpu).reshape(2, 4)
+    y, out = scan_chunk(*(t[:, :0] for t in dev), st)
+    assert y.shape == (2, 0, 4) and torch.equal(out, st)
+    # CPU tensors take the sequential path with the same meaning
+    yc, sc = scan_chunk(x[:, :5], a[:, :5], b[:, :5], c[:, :5])
+    yc2, sc2 = scan_chunk(x[:, 5:], a[:, 5:], b[:, 5:], c[:, 5:], sc)
+    h64, y64 = oracle.forward_f64(x, a, b, c)
+    assert_close("cpu pieces", torch.cat([yc, yc2], 1), y64, 1e-5)
+    assert_close("cpu state", sc2, h64[:, -1], 1e-5)
 
 
 # ---- knobs must not change results ---------------------------------------------------------------------
