@@ -240,6 +240,34 @@ QSSM_API int qssm_scan_backward_carry(const qssm_plan* plan,
                              void* stream);
 
 /*
+ * Gate prologue of the SSM layer: the five projection outputs [rows, S] (row strides ld_* in elements,
+ * so they may be column slices of one wide GEMM output) become the scan's four operands, contiguous
+ * [rows, S] in `out_dtype`, in one pass:
+ *   a = sigmoid(A_pre), x = B_in, c = silu(Ca) * Cb, b = sigmoid(D_pre)
+ * fp32 arithmetic, one rounding per result.  Built pairs (in, out): (f32, f32|f16|bf16), (f16, f16|f32),
+ * (bf16, bf16|f32).  Replaces the elementwise chain of SSM.forward, quick_ssm/layers.py:76-88.
+ */
+QSSM_API int qssm_gates_forward(const void* A_pre, int64_t ld_a, const void* B_in, int64_t ld_b,
+                       const void* Ca, int64_t ld_ca, const void* Cb, int64_t ld_cb,
+                       const void* D_pre, int64_t ld_d,
+                       void* a, void* x, void* c, void* b,
+                       int64_t rows, int32_t S, int32_t in_dtype, int32_t out_dtype, void* stream);
+
+/*
+ * Backward of the gate prologue in one pass: gradients of the scan's operands (contiguous [rows, S] in
+ * `out_dtype`) and the saved projection outputs give the gradients of the projection outputs (contiguous
+ * [rows, S] in `in_dtype`):
+ *   dA_pre = g_a * a (1 - a), dB_in = g_x, dD_pre = g_b * b (1 - b),
+ *   dCa = g_c * Cb * s (1 + Ca (1 - s)), dCb = g_c * Ca * s, with s = sigmoid(Ca).
+ * Replaces what autograd records for quick_ssm/layers.py:76-88.
+ */
+QSSM_API int qssm_gates_backward(const void* g_a, const void* g_x, const void* g_c, const void* g_b,
+                        const void* A_pre, int64_t ld_a, const void* Ca, int64_t ld_ca,
+                        const void* Cb, int64_t ld_cb, const void* D_pre, int64_t ld_d,
+                        void* dA_pre, void* dB_in, void* dCa, void* dCb, void* dD_pre,
+                        int64_t rows, int32_t S, int32_t in_dtype, int32_t out_dtype, void* stream);
+
+/*
  * Streaming copy of `bytes` bytes (16-byte aligned, multiple of 16) on `stream`.  Not part of
  * the scan: it is the known-size kernel against which rocprof's FETCH_SIZE / WRITE_SIZE
  * counters and the achievable-bandwidth ceiling are calibrated by the benchmark.

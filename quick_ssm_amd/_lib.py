@@ -28,6 +28,8 @@ EXPORTED_SYMBOLS = (
     "qssm_scan_backward",
     "qssm_scan_forward_carry",
     "qssm_scan_backward_carry",
+    "qssm_gates_forward",
+    "qssm_gates_backward",
     "qssm_copy_bytes",
 )
 
@@ -110,6 +112,11 @@ def _declare(lib: ctypes.CDLL) -> None:
         [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, vp, vp] + [vp, Strides] * 4
         + [vp, u64, vp, u64, ctypes.c_uint32, vp]
     )
+    i64 = ctypes.c_int64
+    lib.qssm_gates_forward.restype = ctypes.c_int
+    lib.qssm_gates_forward.argtypes = [vp, i64] * 5 + [vp] * 4 + [i64, i32, i32, i32, vp]
+    lib.qssm_gates_backward.restype = ctypes.c_int
+    lib.qssm_gates_backward.argtypes = [vp] * 4 + [vp, i64] * 4 + [vp] * 5 + [i64, i32, i32, i32, vp]
     lib.qssm_copy_bytes.restype = ctypes.c_int
     lib.qssm_copy_bytes.argtypes = [vp, vp, u64, vp]
 

@@ -4,6 +4,9 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <initializer_list>
+#include <utility>
+
 #include "scan_common.h"
 
 namespace qssm {
@@ -458,6 +461,57 @@ int qssm_scan_backward_carry(const qssm_plan* plan, const void* x, qssm_strides 
     return fail(QSSM_EINVAL, "no backward kernel for vec=%d steps=%d threads=%d", plan->vec, plan->steps, plan->threads);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : hip_fail(e, "scan_bwd_kernel launch");
+}
+
+// Widest lane vector (4, 2 or 1 elements) every listed tensor allows.
+static int gate_vec(int S, std::initializer_list<std::pair<const void*, int64_t>> tensors, int elem_bytes_in,
+                    std::initializer_list<const void*> dense, int elem_bytes_dense) {
+  for (int v = 4; v > 1; v >>= 1) {
+    bool ok = S % v == 0;
+    for (const auto& t : tensors) ok = ok && ((uintptr_t)t.first) % (size_t)(v * elem_bytes_in) == 0 && t.second % v == 0;
+    for (const void* d : dense) ok = ok && ((uintptr_t)d) % (size_t)(v * elem_bytes_dense) == 0;
+    if (ok) return v;
+  }
+  return 1;
+}
+
+int qssm_gates_forward(const void* A_pre, int64_t ld_a, const void* B_in, int64_t ld_b, const void* Ca, int64_t ld_ca,
+                       const void* Cb, int64_t ld_cb, const void* D_pre, int64_t ld_d, void* a, void* x, void* c,
+                       void* b, int64_t rows, int32_t S, int32_t in_dtype, int32_t out_dtype, void* stream) {
+  const int es = dtype_size(in_dtype), os = dtype_size(out_dtype);
+  if (es == 0 || os == 0) return fail(QSSM_EINVAL, "unknown dtype code");
+  if (rows < 0 || S < 0) return fail(QSSM_EINVAL, "negative dimension");
+  if (rows == 0 || S == 0) return 0;
+  if (!A_pre || !B_in || !Ca || !Cb || !D_pre || !a || !x || !c || !b) return fail(QSSM_EINVAL, "NULL tensor");
+  if (ld_a < S || ld_b < S || ld_ca < S || ld_cb < S || ld_d < S) return fail(QSSM_EINVAL, "row stride below S");
+  GateFwdArgs args{A_pre, B_in, Ca, Cb, D_pre, ld_a, ld_b, ld_ca, ld_cb, ld_d, a, x, c, b, rows, S};
+  const int vec = gate_vec(S, {{A_pre, ld_a}, {B_in, ld_b}, {Ca, ld_ca}, {Cb, ld_cb}, {D_pre, ld_d}}, es,
+                           {a, x, c, b}, os);
+  if (!launch_gates_any(in_dtype, out_dtype, &args, nullptr, vec, (hipStream_t)stream))
+    return fail(QSSM_EINVAL, "gate dtype pair (in=%d, out=%d) is not built", in_dtype, out_dtype);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : hip_fail(e, "gates_fwd_kernel launch");
+}
+
+int qssm_gates_backward(const void* g_a, const void* g_x, const void* g_c, const void* g_b, const void* A_pre,
+                        int64_t ld_a, const void* Ca, int64_t ld_ca, const void* Cb, int64_t ld_cb, const void* D_pre,
+                        int64_t ld_d, void* dA_pre, void* dB_in, void* dCa, void* dCb, void* dD_pre, int64_t rows,
+                        int32_t S, int32_t in_dtype, int32_t out_dtype, void* stream) {
+  const int es = dtype_size(in_dtype), os = dtype_size(out_dtype);
+  if (es == 0 || os == 0) return fail(QSSM_EINVAL, "unknown dtype code");
+  if (rows < 0 || S < 0) return fail(QSSM_EINVAL, "negative dimension");
+  if (rows == 0 || S == 0) return 0;
+  if (!g_a || !g_x || !g_c || !g_b || !A_pre || !Ca || !Cb || !D_pre || !dA_pre || !dB_in || !dCa || !dCb || !dD_pre)
+    return fail(QSSM_EINVAL, "NULL tensor");
+  if (ld_a < S || ld_ca < S || ld_cb < S || ld_d < S) return fail(QSSM_EINVAL, "row stride below S");
+  GateBwdArgs args{g_a, g_x, g_c, g_b, A_pre, Ca, Cb, D_pre, ld_a, ld_ca, ld_cb, ld_d,
+                   dA_pre, dB_in, dCa, dCb, dD_pre, rows, S};
+  int vec = gate_vec(S, {{A_pre, ld_a}, {Ca, ld_ca}, {Cb, ld_cb}, {D_pre, ld_d}, {dA_pre, S}, {dB_in, S}, {dCa, S},
+                         {dCb, S}, {dD_pre, S}}, es, {g_a, g_x, g_c, g_b}, os);
+  if (!launch_gates_any(in_dtype, out_dtype, nullptr, &args, vec, (hipStream_t)stream))
+    return fail(QSSM_EINVAL, "gate dtype pair (in=%d, out=%d) is not built", in_dtype, out_dtype);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : hip_fail(e, "gates_bwd_kernel launch");
 }
 
 int qssm_copy_bytes(void* dst, const void* src, uint64_t bytes, void* stream) {

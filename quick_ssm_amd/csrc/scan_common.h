@@ -415,4 +415,28 @@ inline size_t bwd_cg_lds_bytes(int nth, int steps) { return (size_t)2 * nth * st
 fwd_launch_fn find_fwd_launcher(int in_dtype, int out_dtype);
 bwd_launch_fn find_bwd_launcher(int in_dtype, int out_dtype);
 
+// ---- gate prologue of the SSM layer (gates.hip) --------------------------------------------------
+
+struct GateFwdArgs {
+  const void *A_pre, *B_in, *Ca, *Cb, *D_pre;  // [rows, S], row strides in elements
+  int64_t ld_a, ld_b, ld_ca, ld_cb, ld_d;
+  void *a, *x, *c, *b;                          // [rows, S] contiguous
+  int64_t rows;
+  int S;
+};
+
+struct GateBwdArgs {
+  const void *g_a, *g_x, *g_c, *g_b;            // [rows, S] contiguous, storage of the scan's operands
+  const void *A_pre, *Ca, *Cb, *D_pre;          // [rows, S], row strides in elements
+  int64_t ld_a, ld_ca, ld_cb, ld_d;
+  void *dA_pre, *dB_in, *dCa, *dCb, *dD_pre;    // [rows, S] contiguous, storage of the projections
+  int64_t rows;
+  int S;
+};
+
+// One entry per (projection storage, operand storage) pair; exactly one of f, b is non-null.
+// Returns false if the pair or vec is not built.
+bool launch_gates_any(int in_dtype, int out_dtype, const GateFwdArgs* f, const GateBwdArgs* b, int vec,
+                      hipStream_t stream);
+
 }  // namespace qssm

@@ -1,8 +1,9 @@
 """`SSM` and `RMSNorm`: the layer that feeds the scan.
 
 Same constructor arguments, parameter names (so state dicts interchange) and forward keywords as
-the reference's quick_ssm/layers.py:9-107.  The projections and gate activations stay on torch
-GEMMs / elementwise ops; only the scan inside is the HIP path.  Roles of the projections
+the reference's quick_ssm/layers.py:9-107.  The projections stay on torch GEMMs; the gate
+activations and casts between them and the scan are one fused HIP pass (quick_ssm_amd/gates.py),
+and the scan is the HIP path.  Roles of the projections
 (quick_ssm/test_swiglu_equiv.py:60-70): A_proj -> forget gate a, B_proj -> the scan's input x,
 D_proj -> input gate b, C_proj_a/C_proj_b -> SwiGLU output gate c, out_proj -> output.
 """
@@ -12,8 +13,8 @@ from typing import Optional
 
 import torch
 import torch.nn as nn
-import torch.nn.functional as F
 
+from .gates import gate_prologue
 from .scan_interface import scan
 
 
@@ -65,11 +66,8 @@ class SSM(nn.Module):
 
     def gates(self, u: torch.Tensor):
         """The scan's four operands (x, a, b, c) from the normalised input, in `compute_dtype`."""
-        dt = self.compute_dtype
-        forget = torch.sigmoid(self.A_proj(u)).to(dt)
-        drive = self.B_proj(u).to(dt)
-        out_gate = (F.silu(self.C_proj_a(u)) * self.C_proj_b(u)).to(dt)
-        in_gate = torch.sigmoid(self.D_proj(u)).to(dt)
+        forget, drive, out_gate, in_gate = gate_prologue(
+            self.A_proj(u), self.B_proj(u), self.C_proj_a(u), self.C_proj_b(u), self.D_proj(u), self.compute_dtype)
         return drive, forget, in_gate, out_gate
 
     def forward(

@@ -177,6 +177,43 @@ def test_carried_state_gradients_by_finite_differences():
     np.testing.assert_array_equal(oracle.backward_carry_f64(e, e, e, e, e, h0, g_final)[4], g_final.astype(np.float64))
 
 
+def test_gate_oracle_against_torch_library_routines_and_differences():
+    # Pins oracle/gates_oracle.py: forward against torch.sigmoid / silu in float64, backward against torch's autograd
+    # of those library routines and against central differences of the float64 forward.
+    from oracle import gates_oracle
+    import torch.nn.functional as F
+    gen = torch.Generator().manual_seed(17)
+    z = [(torch.randn(3, 7, 5, generator=gen, dtype=torch.float64) * 3).requires_grad_(True) for _ in range(5)]
+    g = [torch.randn(3, 7, 5, generator=gen, dtype=torch.float64) for _ in range(4)]
+    a, x, c, b = torch.sigmoid(z[0]), z[1] * 1.0, F.silu(z[2]) * z[3], torch.sigmoid(z[4])
+    got = gates_oracle.gates_forward_f64(*z)
+    for name, mine, lib in zip("axcb", got, (a, x, c, b)):
+        np.testing.assert_allclose(mine, lib.detach().numpy(), rtol=1e-14, atol=1e-16, err_msg=name)
+    (a * g[0] + x * g[1] + c * g[2] + b * g[3]).sum().backward()
+    grads = gates_oracle.gates_backward_f64(*g, z[0], z[2], z[3], z[4])
+    for name, mine, leaf in zip(("dA", "dB", "dCa", "dCb", "dD"), grads, z):
+        np.testing.assert_allclose(mine, leaf.grad.numpy(), rtol=1e-12, atol=1e-15, err_msg=name)
+    # central differences on one element of every input
+    zs = [t.detach().numpy().copy() for t in z]
+    gs = [t.numpy() for t in g]
+
+    def loss(vals):
+        out = gates_oracle.gates_forward_f64(*vals)
+        return sum(float((o * w).sum()) for o, w in zip(out, gs))
+
+    for k in range(5):
+        bump = [v.copy() for v in zs]
+        lo = [v.copy() for v in zs]
+        bump[k][1, 2, 3] += 1e-6
+        lo[k][1, 2, 3] -= 1e-6
+        fd = (loss(bump) - loss(lo)) / 2e-6
+        assert abs(fd - grads[k][1, 2, 3]) <= 1e-7 * max(1.0, abs(fd))
+    # saturation: large |z| must not overflow
+    big = np.array([[-800.0, 800.0]])
+    sat = gates_oracle.gates_forward_f64(big, big, big, big, big)
+    assert np.all(np.isfinite(sat[0])) and sat[0][0, 0] == 0.0 and sat[0][0, 1] == 1.0 and sat[2][0, 0] == 0.0
+
+
 def test_c_and_torch_flavours_agree_bitwise_in_fp32():
     x, a, b, c, dy = make_inputs((2, 130, 5), seed=3)
     h_c = oracle.forward_f32_seq(x, a, b)
