@@ -121,15 +121,22 @@ QSSM_API int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, i
  * Two device buffers accompany every launch, both owned by the caller and both zero-filled
  * (qssm_zero_fill) when they are allocated:
  *
- *   control    status word + one ticket counter per chain (plan.control_bytes).  A launch needs it
- *              zero on entry and leaves it zero, except that the status word becomes nonzero if
- *              a tile gave up waiting for a neighbour (the outputs of that launch are then
- *              poisoned with NaN and the buffer must be zero-filled again).
+ *   control    status word, a launch count and one ticket counter per chain (plan.control_bytes).
+ *              A launch needs the status word and the ticket counters zero on entry and leaves them
+ *              zero, except that the status word becomes nonzero if a tile gave up waiting for a
+ *              neighbour (the outputs of that launch are then poisoned with NaN and the buffer
+ *              must be zero-filled again).
  *   workspace  the words tiles hand to each other (plan.workspace_bytes; may be 0).  Words are
- *              tagged with the launch's `epoch`, so nothing has to be cleared between launches:
+ *              tagged with the launch's epoch, so nothing has to be cleared between launches:
  *              zero-fill it once, and again before an epoch value would be reused.
  *
- * Launches that share these buffers must be ordered on one stream and carry different epochs.
+ * Launches that share these buffers must be ordered on one stream and carry different epochs.  Two
+ * ways to number them; use one per pair of buffers from zero-fill to zero-fill:
+ *   epoch != 0   the caller counts (1, 2, 3, ...).
+ *   epoch == 0   the library counts in the control block: the launch reads its epoch from device
+ *                memory and a one-lane kernel behind it adds one.  Nothing launch-specific is then
+ *                baked into kernel arguments, so launches captured in a HIP graph replay correctly
+ *                (the count wraps after 2^32 - 1 launches; zero-fill the workspace before that).
  */
 
 /* Zero-fill a buffer with a fill kernel on `stream` (safe under graph capture; no hipMemset). */
@@ -145,8 +152,9 @@ QSSM_API int qssm_control_status(const void* control, void* stream, int32_t* sta
  *   y          may be NULL (state-only pass: only `ckpt` is produced).
  *   h_out      optional fp32 [B, L, D] (strides sh): every h(t); the checkpoint=False case.
  *   ckpt       optional fp32 [B, n_ckpt, D] contiguous: h(t-1) at t = k * ckpt_stride.
- *   epoch      nonzero, and different from the epoch of every earlier launch that used this
- *              workspace since it was last zero-filled (a per-workspace counter does it).
+ *   epoch      0 (the library counts launches in the control block), or a nonzero value different
+ *              from the epoch of every earlier launch that used this workspace since it was last
+ *              zero-filled (a per-workspace counter does it).
  *   control, workspace: see above.
  * Replaces _TritonScanFunction.forward's per-tile body (quick_ssm/scan_interface.py:91-107):
  * block_scan_forward_3d (quick_ssm/triton_forwards.py:134-172, three launches + fp32 scratch)

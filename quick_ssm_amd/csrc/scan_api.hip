@@ -127,6 +127,15 @@ static bool tile_span_ok(const qssm_plan* pl, const void* p, int64_t sb, int64_t
   return span < ((int64_t)1 << 31);
 }
 
+// One lane behind every launch that uses device-counted epochs: the next launch on the stream gets
+// the next flag value.  A kernel of its own, so that every workgroup of the scan has read the
+// count before it changes, and so that a captured graph replays correctly (the count lives in device
+// memory, not in a kernel argument).  The count never takes the value whose successor is zero.
+__global__ void count_launch_kernel(unsigned* count) {
+  const unsigned next = *count + 1u;
+  *count = next == 0xffffffffu ? 0u : next;
+}
+
 static void fill_geometry(Geometry* g, const qssm_plan* pl, void* control, void* workspace, uint32_t epoch) {
   g->B = pl->B;
   g->L = pl->L;
@@ -141,6 +150,8 @@ static void fill_geometry(Geometry* g, const qssm_plan* pl, void* control, void*
   g->ckpt_stride = pl->ckpt_stride;
   g->n_ckpt = pl->n_ckpt;
   g->epoch = epoch;
+  // epoch 0: the launches are counted in the control block itself (see count_launch_kernel)
+  g->launch_count = epoch != 0 ? nullptr : (const unsigned*)((const char*)control + kLaunchCountOffset);
   char* ws = (char*)workspace;
   g->status = (int*)control;
   g->tickets = (unsigned*)((char*)control + kStatusBytes);
@@ -359,7 +370,6 @@ int qssm_scan_forward_carry(const qssm_plan* plan, const void* x, qssm_strides s
   if (((uintptr_t)control) % 8 != 0 || ((uintptr_t)workspace) % 8 != 0)
     return fail(QSSM_EALIGN, "control block and workspace must be 8-byte aligned");
 
-  if (epoch == 0) return fail(QSSM_EINVAL, "epoch must be nonzero");
   if (!tile_span_ok(plan, x, sx.b, sx.l, es) || !tile_span_ok(plan, a, sa.b, sa.l, es) ||
       !tile_span_ok(plan, b, sb.b, sb.l, es) || !tile_span_ok(plan, c, sc.b, sc.l, es) ||
       !tile_span_ok(plan, y, sy.b, sy.l, os) || !tile_span_ok(plan, h_out, sh.b, sh.l, 4))
@@ -383,6 +393,9 @@ int qssm_scan_forward_carry(const qssm_plan* plan, const void* x, qssm_strides s
   if (c_in_lds) lds += fwd_c_lds_bytes(plan->threads, plan->steps);
   if (!fn(args, plan->vec, plan->steps, plan->threads, c_in_lds, grid, lds, (hipStream_t)stream))
     return fail(QSSM_EINVAL, "no forward kernel for vec=%d steps=%d threads=%d", plan->vec, plan->steps, plan->threads);
+  if (epoch == 0 && plan->n_seg > 1)
+    hipLaunchKernelGGL(count_launch_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream,
+                       (unsigned*)((char*)control + kLaunchCountOffset));
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : hip_fail(e, "scan_fwd_kernel launch");
 }
@@ -430,7 +443,6 @@ int qssm_scan_backward_carry(const qssm_plan* plan, const void* x, qssm_strides 
   if (((uintptr_t)control) % 8 != 0 || ((uintptr_t)workspace) % 8 != 0)
     return fail(QSSM_EALIGN, "control block and workspace must be 8-byte aligned");
 
-  if (epoch == 0) return fail(QSSM_EINVAL, "epoch must be nonzero");
   if (!tile_span_ok(plan, x, sx.b, sx.l, es) || !tile_span_ok(plan, a, sa.b, sa.l, es) ||
       !tile_span_ok(plan, b, sb.b, sb.l, es) || !tile_span_ok(plan, c, sc.b, sc.l, es) ||
       !tile_span_ok(plan, dy, sdy.b, sdy.l, os) || !tile_span_ok(plan, dx, sdx.b, sdx.l, es) ||
@@ -459,6 +471,9 @@ int qssm_scan_backward_carry(const qssm_plan* plan, const void* x, qssm_strides 
   if (cg_in_lds) lds += bwd_cg_lds_bytes(plan->threads, plan->steps);
   if (!fn(args, plan->vec, plan->steps, plan->threads, cg_in_lds, grid, lds, (hipStream_t)stream))
     return fail(QSSM_EINVAL, "no backward kernel for vec=%d steps=%d threads=%d", plan->vec, plan->steps, plan->threads);
+  if (epoch == 0 && plan->n_seg > 1)
+    hipLaunchKernelGGL(count_launch_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream,
+                       (unsigned*)((char*)control + kLaunchCountOffset));
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : hip_fail(e, "scan_bwd_kernel launch");
 }

@@ -37,6 +37,8 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   const int NG = NTH >> g.g_log2;
   const int cols = G * VEC;
   const int R = g.cluster;
+  // Flag value of this launch: the host's, or one more than the launches counted in the control block.
+  const unsigned epoch = g.launch_count != nullptr ? *g.launch_count + 1u : g.epoch;
   float* sA = lds;                       // [NTH * VEC] per-lane map, multiplier (both directions)
   float* sXf = sA + NTH * VEC;           // [NTH * VEC] forward offset
   float* sXe = sXf + NTH * VEC;          // [NTH * VEC] reverse offset
@@ -222,7 +224,7 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
 #pragma unroll
     for (int v = 0; v < VEC; ++v) ein[v] = ev.v[v];
   }
-  if (want_state && pk_state.ready(g.epoch)) {
+  if (want_state && pk_state.ready(epoch)) {
     state_here = true;
 #pragma unroll
     for (int v = 0; v < VEC; ++v) ein[v] = pk_state.value(v);
@@ -320,13 +322,13 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
         unsigned long long* mw = g.maps + ((int64_t)chain * g.n_seg + seg) * cols * 2 + lane;
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
-          word_publish(mw + (2 * v) * G, g.epoch, At[v]);
-          word_publish(mw + (2 * v + 1) * G, g.epoch, Xt[v]);
+          word_publish(mw + (2 * v) * G, epoch, At[v]);
+          word_publish(mw + (2 * v + 1) * G, epoch, Xt[v]);
         }
       }
     }
     // The second look's answers.
-    if (ask_state && pk_state.ready(g.epoch)) {
+    if (ask_state && pk_state.ready(epoch)) {
       state_here = true;
 #pragma unroll
       for (int v = 0; v < VEC; ++v) ein[v] = pk_state.value(v);
@@ -338,7 +340,7 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
       if (dok && !(i == j && map_here)) {
         float w[2 * VEC];
         const unsigned long long* mw = g.maps + ((int64_t)chain * g.n_seg + (seg + 1 + i)) * cols * 2 + lane;
-        if (!words_wait<2 * VEC>(mw, G, g.epoch, w, kPollSlow)) raise_status(g.status, 1);
+        if (!words_wait<2 * VEC>(mw, G, epoch, w, kPollSlow)) raise_status(g.status, 1);
         float wa[VEC], wx[VEC];
 #pragma unroll
         for (int v = 0; v < VEC; ++v) { wa[v] = w[2 * v]; wx[v] = w[2 * v + 1]; }
@@ -347,7 +349,7 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
       }
     }
     if (want_state && !state_here) {
-      if (!words_wait<VEC>(next_state, G, g.epoch, ein, m == 0 ? kPollChain : kPollUrgent)) raise_status(g.status, 1);
+      if (!words_wait<VEC>(next_state, G, epoch, ein, m == 0 ? kPollChain : kPollUrgent)) raise_status(g.status, 1);
     }
     if (cnt > 0) lds_barrier();
     if (edge) {
@@ -361,7 +363,7 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
       if (dok && m == 0 && s > 0) {
         unsigned long long* sw = g.states + ((int64_t)chain * g.n_super + s) * cols + lane;
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) word_publish(sw + v * G, g.epoch, At[v] * ein[v] + Xt[v]);
+        for (int v = 0; v < VEC; ++v) word_publish(sw + v * G, epoch, At[v] * ein[v] + Xt[v]);
       }
       lds_put<VEC>(sE + dl, ein);
     }

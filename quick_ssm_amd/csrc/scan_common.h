@@ -44,10 +44,13 @@ namespace qssm {
 // in total.
 constexpr int kSpinLimit = 1 << 20;
 
-// Control block layout (bytes): [0,64) status word; then one 64-byte slot per chain holding its
+// Control block layout (bytes): [0,4) status word, [4,8) launches counted on the device (the epoch
+// of a launch whose host passes epoch 0 is this count + 1; a one-lane kernel behind the launch
+// adds one), rest of the first 64 bytes unused; then one 64-byte slot per chain holding its
 // ticket counter.  Workspace layout: the tile maps (2 words per column per tile), then,
 // 256-byte aligned, the cluster states (1 word per column per cluster).
 constexpr uint64_t kStatusBytes = 64;
+constexpr uint64_t kLaunchCountOffset = 4;
 constexpr uint64_t kTicketStride = 64;
 
 __host__ __device__ inline uint64_t ws_align(uint64_t off) { return (off + 255u) & ~uint64_t(255); }
@@ -362,7 +365,8 @@ struct Geometry {
   int n_super;      // clusters per chain
   int ckpt_stride;  // spacing of saved states
   int n_ckpt;       // saved states per (batch, column)
-  unsigned epoch;   // this launch's flag value (nonzero)
+  unsigned epoch;   // this launch's flag value (nonzero), when the host counts launches
+  const unsigned* launch_count;  // else: launches counted on the device; the flag value is *launch_count + 1
   int* status;
   unsigned* tickets;
   unsigned long long* maps;    // [chain][tile][2 * VEC planes][G lanes]: the tile's affine map (A, X)

@@ -28,6 +28,8 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   const int NG = NTH >> g.g_log2;
   const int cols = G * VEC;
   const int R = g.cluster;
+  // Flag value of this launch: the host's, or one more than the launches counted in the control block.
+  const unsigned epoch = g.launch_count != nullptr ? *g.launch_count + 1u : g.epoch;
   float* sA = lds;                       // [NTH * VEC] per-lane map, multiplier
   float* sX = sA + NTH * VEC;            // [NTH * VEC] per-lane map, offset
   float* sPA = sX + NTH * VEC;           // [(R-1) * cols] maps of the earlier tiles of the cluster
@@ -157,7 +159,7 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
 #pragma unroll
     for (int v = 0; v < VEC; ++v) hin[v] = hv.v[v];
   }
-  if (want_map && pk_map.ready(g.epoch)) {
+  if (want_map && pk_map.ready(epoch)) {
     map_here = true;
     float wa[VEC], wx[VEC];
 #pragma unroll
@@ -165,7 +167,7 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
     lds_put<VEC>(sPA + j * cols + dl, wa);
     lds_put<VEC>(sPX + j * cols + dl, wx);
   }
-  if (want_state && pk_state.ready(g.epoch)) {
+  if (want_state && pk_state.ready(epoch)) {
     state_here = true;
 #pragma unroll
     for (int v = 0; v < VEC; ++v) hin[v] = pk_state.value(v);
@@ -232,13 +234,13 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
         unsigned long long* mw = g.maps + ((int64_t)chain * g.n_seg + seg) * cols * 2 + lane;
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
-          word_publish(mw + (2 * v) * G, g.epoch, At[v]);
-          word_publish(mw + (2 * v + 1) * G, g.epoch, Xt[v]);
+          word_publish(mw + (2 * v) * G, epoch, At[v]);
+          word_publish(mw + (2 * v + 1) * G, epoch, Xt[v]);
         }
       }
     }
     // The second look's answers.
-    if (ask_map && pk_map.ready(g.epoch)) {
+    if (ask_map && pk_map.ready(epoch)) {
       map_here = true;
       float wa[VEC], wx[VEC];
 #pragma unroll
@@ -246,7 +248,7 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
       lds_put<VEC>(sPA + j * cols + dl, wa);
       lds_put<VEC>(sPX + j * cols + dl, wx);
     }
-    if (ask_state && pk_state.ready(g.epoch)) {
+    if (ask_state && pk_state.ready(epoch)) {
       state_here = true;
 #pragma unroll
       for (int v = 0; v < VEC; ++v) hin[v] = pk_state.value(v);
@@ -258,7 +260,7 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
       if (dok && !(i == j && map_here)) {
         float w[2 * VEC];
         const unsigned long long* mw = g.maps + ((int64_t)chain * g.n_seg + (seg - m + i)) * cols * 2 + lane;
-        if (!words_wait<2 * VEC>(mw, G, g.epoch, w, kPollSlow)) raise_status(g.status, 1);
+        if (!words_wait<2 * VEC>(mw, G, epoch, w, kPollSlow)) raise_status(g.status, 1);
         float wa[VEC], wx[VEC];
 #pragma unroll
         for (int v = 0; v < VEC; ++v) { wa[v] = w[2 * v]; wx[v] = w[2 * v + 1]; }
@@ -267,7 +269,7 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
       }
     }
     if (want_state && !state_here) {
-      if (!words_wait<VEC>(prev_state, G, g.epoch, hin, m == R - 1 ? kPollChain : kPollUrgent)) raise_status(g.status, 1);
+      if (!words_wait<VEC>(prev_state, G, epoch, hin, m == R - 1 ? kPollChain : kPollUrgent)) raise_status(g.status, 1);
     }
     if (m > 0) lds_barrier();
     if (edge) {
@@ -281,7 +283,7 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
       if (dok && m == R - 1 && s + 1 < g.n_super) {
         unsigned long long* sw = g.states + ((int64_t)chain * g.n_super + s) * cols + lane;
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) word_publish(sw + v * G, g.epoch, At[v] * hin[v] + Xt[v]);
+        for (int v = 0; v < VEC; ++v) word_publish(sw + v * G, epoch, At[v] * hin[v] + Xt[v]);
       }
       lds_put<VEC>(sH + dl, hin);
     }

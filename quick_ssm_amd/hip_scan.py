@@ -32,7 +32,7 @@ _EPOCH_MAX = 0xFFFFFFFF
 
 
 class _Buffers:
-    """Per (device, stream): the control block, the workspace and the epoch counter that goes with it."""
+    """Per (device, stream, who numbers the launches): control block, workspace, and the host's launch count."""
 
     __slots__ = ("control", "workspace", "epoch")
 
@@ -42,7 +42,7 @@ class _Buffers:
         self.epoch = 0
 
 
-_buffers: Dict[Tuple[int, int], _Buffers] = {}
+_buffers: Dict[Tuple[int, int, bool], _Buffers] = {}
 
 
 def kernel_dtypes(in_dtypes: Sequence[torch.dtype], out_dtype: torch.dtype) -> Tuple[torch.dtype, torch.dtype]:
@@ -95,41 +95,82 @@ def _align_elems(tensors: Sequence[Optional[Tensor]], D: int) -> int:
     return 1
 
 
+_device_counted = threading.local()
+
+
+class device_counted_launches:
+    """Context manager: scan launches inside number themselves in their control block (epoch argument 0), as
+    launches recorded into a graph do, and use the buffers kept for such launches.
+
+    Launches being recorded into a graph do this by themselves, but cannot allocate: run the work once inside this
+    context, on the stream that will capture, and the control block and workspace exist (large enough) when the
+    capture starts.
+    """
+
+    def __enter__(self):
+        self._old = getattr(_device_counted, "on", False)
+        _device_counted.on = True
+        return self
+
+    def __exit__(self, *exc):
+        _device_counted.on = self._old
+        return False
+
+
 def _launch_buffers(device: torch.device, stream: int, plan: Plan) -> Tuple[Tensor, Tensor, int]:
-    """Control block, workspace and epoch for the next launch on (device, stream).
+    """Control block, workspace and epoch argument for the next launch on (device, stream).
 
     Both buffers are zero-filled when they are allocated (torch.zeros runs a fill kernel on the
-    current stream, ahead of the launch that uses them) and grown on demand.  The control block is
-    left zero by every launch.  The workspace is never cleared: every launch gets the next epoch
-    value, and when the 32-bit counter is used up the workspace is replaced by a fresh zeroed one.
+    current stream, ahead of the launch that uses them) and grown on demand.  Every launch leaves
+    the control block's status word and ticket counters zero.  The workspace is never cleared:
+    every launch gets the next epoch.  Eager launches are numbered here.  Launches recorded into a
+    graph (and those inside `device_counted_launches`) use a pair of buffers of their own and are
+    numbered in the control block itself (epoch argument 0), so that replays number themselves, at
+    the price of a one-lane counting kernel behind each launch.  A workspace that has to grow, or
+    whose 32-bit host numbering is used up, is replaced by a fresh zeroed one.
     """
-    key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
+    capturing = bool(torch.cuda.is_current_stream_capturing())
+    on_device = capturing or getattr(_device_counted, "on", False)
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream, on_device)
     with _ws_lock:
         buf = _buffers.get(key)
         if buf is None:
-            buf = _buffers[key] = _Buffers()
+            buf = _Buffers()
         need_c, need_w = int(plan.control_bytes), max(int(plan.workspace_bytes), 256)
-        if buf.control is None or buf.control.numel() < need_c:
+        grow_c = buf.control is None or buf.control.numel() < need_c
+        grow_w = grow_c or buf.workspace is None or buf.workspace.numel() < need_w or buf.epoch >= _EPOCH_MAX
+        if capturing and grow_w:
+            raise RuntimeError(
+                "quick_ssm_amd: a scan launch being recorded into a graph cannot allocate its control block and "
+                "workspace; run the same work once inside `hip_scan.device_counted_launches()` on this stream first")
+        _buffers[key] = buf
+        if grow_c:
+            # a new control block restarts the device-side count: the workspace must not keep words of the old numbering
             buf.control = torch.zeros(max(1 << 16, 1 << (need_c - 1).bit_length()), dtype=torch.uint8, device=device)
-        if buf.workspace is None or buf.workspace.numel() < need_w or buf.epoch >= _EPOCH_MAX:
+        if grow_w:
             buf.workspace = torch.zeros(max(1 << 20, 1 << (need_w - 1).bit_length()), dtype=torch.uint8, device=device)
             buf.epoch = 0
+        if on_device:
+            return buf.control, buf.workspace, 0
         buf.epoch += 1
         return buf.control, buf.workspace, buf.epoch
 
 
 def workspace_status(device: Optional[torch.device] = None) -> int:
-    """Status word of the current stream's control block (synchronises).  0 = all launches completed."""
+    """Status words of the current stream's control blocks, or-ed (synchronises).  0 = all launches completed."""
     device = torch.device("cuda", torch.cuda.current_device()) if device is None else device
     stream = torch.cuda.current_stream(device).cuda_stream
-    key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
-    with _ws_lock:
-        buf = _buffers.get(key)
-    if buf is None or buf.control is None:
-        return 0
-    out = ctypes.c_int32(0)
-    _lib.check(_lib.load().qssm_control_status(buf.control.data_ptr(), stream, ctypes.byref(out)))
-    return int(out.value)
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    status = 0
+    for on_device in (False, True):
+        with _ws_lock:
+            buf = _buffers.get((index, stream, on_device))
+        if buf is None or buf.control is None:
+            continue
+        out = ctypes.c_int32(0)
+        _lib.check(_lib.load().qssm_control_status(buf.control.data_ptr(), stream, ctypes.byref(out)))
+        status |= int(out.value)
+    return status
 
 
 def reset_workspaces() -> None:

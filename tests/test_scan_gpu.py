@@ -316,6 +316,94 @@ def test_carried_state_argument_errors_and_empty_piece(gpu):
     assert_close("cpu state", sc2, h64[:, -1], 1e-5)
 
 
+# ---- launch numbering: by the caller, by the library, and under graph replay --------------------------------
+
+def test_c_abi_with_caller_counted_epochs(gpu):
+    # the raw C ABI the way INTEGRATION.md shows it: own control block and workspace, epochs 1, 2, 3 from the caller
+    import ctypes
+    lib = _lib.load()
+    shape = (2, 900, 256)
+    x, a, b, c, dy = make_inputs(shape, dtype=torch.bfloat16, seed=51)
+    ref = oracle_all(x, a, b, c, dy)
+    ops = [t.to(gpu).contiguous() for t in (x, a, b, c, dy)]
+    B, L, D = shape
+    tune = 7 | (8 << 8)
+    bwd = hip_scan.make_plan(B, L, D, torch.bfloat16, torch.bfloat16, _lib.QSSM_BACKWARD, 8, 0, tune)
+    fwd = hip_scan.make_plan(B, L, D, torch.bfloat16, torch.bfloat16, _lib.QSSM_FORWARD, 8, bwd.seg_len, tune)
+    assert fwd.n_seg > 1 and bwd.n_seg > 1
+    control = torch.zeros(max(fwd.control_bytes, bwd.control_bytes), dtype=torch.uint8, device=gpu)
+    workspace = torch.zeros(max(fwd.workspace_bytes, bwd.workspace_bytes), dtype=torch.uint8, device=gpu)
+    stream = torch.cuda.current_stream().cuda_stream
+    st = lambda t: _lib.Strides(t.stride(0), t.stride(1))
+    none = _lib.Strides(0, 0)
+    epoch = 0
+    for _ in range(3):  # same buffers, next epochs: old words must read as "not there yet"
+        y = torch.empty(shape, dtype=torch.bfloat16, device=gpu)
+        ckpt = torch.empty(B, fwd.n_ckpt, D, dtype=torch.float32, device=gpu)
+        grads = [torch.empty(shape, dtype=torch.bfloat16, device=gpu) for _ in range(4)]
+        epoch += 1
+        _lib.check(lib.qssm_scan_forward(
+            ctypes.byref(fwd), ops[0].data_ptr(), st(ops[0]), ops[1].data_ptr(), st(ops[1]), ops[2].data_ptr(), st(ops[2]),
+            ops[3].data_ptr(), st(ops[3]), y.data_ptr(), st(y), None, none, ckpt.data_ptr(),
+            control.data_ptr(), control.numel(), workspace.data_ptr(), workspace.numel(), epoch, stream))
+        epoch += 1
+        _lib.check(lib.qssm_scan_backward(
+            ctypes.byref(bwd), ops[0].data_ptr(), st(ops[0]), ops[1].data_ptr(), st(ops[1]), ops[2].data_ptr(), st(ops[2]),
+            ops[3].data_ptr(), st(ops[3]), ops[4].data_ptr(), st(ops[4]), None, none, ckpt.data_ptr(),
+            grads[0].data_ptr(), st(grads[0]), grads[1].data_ptr(), st(grads[1]), grads[2].data_ptr(), st(grads[2]),
+            grads[3].data_ptr(), st(grads[3]),
+            control.data_ptr(), control.numel(), workspace.data_ptr(), workspace.numel(), epoch, stream))
+        status = ctypes.c_int32(-1)
+        _lib.check(lib.qssm_control_status(control.data_ptr(), stream, ctypes.byref(status)))
+        assert status.value == 0
+        got = {"y": y.cpu(), "dx": grads[0].cpu(), "da": grads[1].cpu(), "db": grads[2].cpu(), "dc": grads[3].cpu()}
+        _check_all(got, ref, TOL[torch.bfloat16])
+    assert int(control.view(torch.int32)[1]) == 0   # the library's own count was never used
+
+
+def test_captured_launches_replay_with_new_inputs(gpu):
+    # Forward and backward captured in one graph; every replay reads its epoch from device memory, so tiles of a
+    # replay never mistake the previous replay's words for their neighbours'.  Replays alternate with eager launches
+    # on the same buffers and with new input values, and each one is checked against the eager result.
+    shape = (2, 1500, 512)
+    tune = 7 | (8 << 8)
+    side = torch.cuda.Stream()
+    sets = [make_inputs(shape, dtype=torch.bfloat16, seed=60 + k) for k in range(3)]
+    static = [t.to(gpu).contiguous() for t in sets[0]]
+
+    def run():
+        y, _, ckpt, stride = hip_scan.scan_forward(*static[:4], out_dtype=torch.bfloat16, tune=tune, bwd_tune=tune)
+        return (y,) + tuple(hip_scan.scan_backward(*static, ckpt=ckpt, ckpt_stride=stride, tune=tune))
+
+    with torch.cuda.stream(side):
+        with pytest.raises(RuntimeError):   # recording the very first launch would have to allocate
+            with torch.cuda.graph(torch.cuda.CUDAGraph(), stream=side):
+                run()
+        with hip_scan.device_counted_launches():   # warm-up: the buffers of captured launches exist afterwards
+            run()
+        run()
+        side.synchronize()
+        plan = hip_scan.make_plan(*shape, torch.bfloat16, torch.bfloat16, _lib.QSSM_BACKWARD, 8, 0, tune)
+        assert plan.n_seg > 1 and plan.n_super > 1
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            outs = run()
+    for k in (1, 2, 0, 1):
+        for dst, src in zip(static, sets[k]):
+            dst.copy_(src.to(gpu))
+        with torch.cuda.stream(side):
+            side.wait_stream(torch.cuda.current_stream())
+            eager = [t.clone() for t in run()]      # eager launch between the replays, same buffers
+            graph.replay()
+            side.synchronize()
+            assert hip_scan.workspace_status() == 0
+        ref = oracle_all(*sets[k])
+        got = dict(zip(("y", "dx", "da", "db", "dc"), (t.cpu() for t in outs)))
+        _check_all(got, ref, TOL[torch.bfloat16])
+        for name, g_, e_ in zip(("y", "dx", "da", "db", "dc"), outs, eager):
+            assert torch.equal(g_, e_), name
+
+
 # ---- knobs must not change results ---------------------------------------------------------------------
 
 def test_checkpoint_false_keeps_fp32_states_and_matches(gpu):
