@@ -112,8 +112,13 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   const bool tile_full = (t_tile + g.seg_len <= g.L) && ((strip + 1) * cols <= g.D);
   if (tile_full) {
     if (CLDS) {
+      // register operands first: the forward fold can start on them while c and dy are still on their way
 #pragma unroll
-      for (int i = 0; i < T; ++i) ra[i] = load_stream<Tin, VEC>(ab, ao + i * as);
+      for (int i = 0; i < T; ++i) {
+        ra[i] = load_stream<Tin, VEC>(ab, ao + i * as);
+        rb[i] = load_stream<Tin, VEC>(bb, bo + i * bs);
+        rx[i] = load_stream<Tin, VEC>(xb, xo + i * xs);
+      }
       // lanes 0-31 fetch one row of the strip (16 bytes each), lanes 32-63 the next one
       const int wl = tid & 63;
       const char* csrc = cb + (uint32_t)(j * T + (wl >> 5)) * cs + (uint32_t)(wl & 31) * 16u;
@@ -130,11 +135,11 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
         rc[i] = load_stream<Tin, VEC>(cb, co + i * cs);
         rg[i] = load_stream<Tout, VEC>(gb, go + i * gs);
       }
-    }
 #pragma unroll
-    for (int i = 0; i < T; ++i) {
-      rb[i] = load_stream<Tin, VEC>(bb, bo + i * bs);
-      rx[i] = load_stream<Tin, VEC>(xb, xo + i * xs);
+      for (int i = 0; i < T; ++i) {
+        rb[i] = load_stream<Tin, VEC>(bb, bo + i * bs);
+        rx[i] = load_stream<Tin, VEC>(xb, xo + i * xs);
+      }
     }
   } else {
     // Steps past L and columns past D act as the identity map (a = 1, everything else 0).

@@ -196,10 +196,6 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
 #pragma unroll
   for (int i = 0; i < T; ++i) { forget(ra[i]); forget(rb[i]); forget(rx[i]); }
   lds_barrier();
-  // The loads that write c into LDS are tracked by the vector memory counter only; this wave is the
-  // only reader of the rows it fetched.  Waiting here, before any store of the tile is issued, waits
-  // for nothing but loads.
-  if (CLDS) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   // ---- compose the maps of the lane groups before this one ------------------------------------
   float Ap[VEC], Xp[VEC];
@@ -216,6 +212,11 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
       Ap[v] = ak[v] * Ap[v];
     }
   }
+
+  // The loads that write c into LDS are tracked by the vector memory counter only; this wave is the
+  // only reader of the rows it fetched.  Waiting here, before any store of the tile is issued, waits
+  // for nothing but loads, and c, asked for last, has had the fold above to arrive.
+  if (CLDS) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   // ---- state entering the tile ------------------------------------------------------------------
   if (multi) {
