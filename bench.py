@@ -204,7 +204,8 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": {"float32": "f32", "float16": "f16", "bfloat16": "bf16"}[dt_name] + " storage, f32 arithmetic",
+        # the arithmetic type the path computes in; storage of the operands noted beside it
+        "dtype": "f32 (" + {"float32": "f32", "float16": "f16", "bfloat16": "bf16"}[dt_name] + " storage)",
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: gated linear scan fwd+bwd through scan(), {desc}, "
                                f"block_l={block_l}, checkpoint=True", "B": B, "L": L, "D": D},
