@@ -361,6 +361,43 @@ def test_c_abi_with_caller_counted_epochs(gpu):
     assert int(control.view(torch.int32)[1]) == 0   # the library's own count was never used
 
 
+def test_dirty_control_block_is_reported_and_zero_fill_recovers(gpu):
+    # A control block that is not zero on entry (here: ticket counters far past the end) makes every workgroup leave
+    # at once with status 2 instead of touching memory it does not own; after qssm_zero_fill the same buffers work.
+    import ctypes
+    lib = _lib.load()
+    shape = (1, 600, 256)
+    x, a, b, c, dy = make_inputs(shape, dtype=torch.float16, seed=71)
+    ops = [t.to(gpu).contiguous() for t in (x, a, b, c)]
+    B, L, D = shape
+    plan = hip_scan.make_plan(B, L, D, torch.float16, torch.float16, _lib.QSSM_FORWARD, 8, 0, 7 | (8 << 8))
+    assert plan.n_seg > 1
+    control = torch.zeros(plan.control_bytes, dtype=torch.uint8, device=gpu)
+    workspace = torch.zeros(plan.workspace_bytes, dtype=torch.uint8, device=gpu)
+    control.view(torch.int32)[16:] = 0x7fff0000           # every ticket slot; the status word stays zero
+    stream = torch.cuda.current_stream().cuda_stream
+    st = lambda t: _lib.Strides(t.stride(0), t.stride(1))
+    none = _lib.Strides(0, 0)
+
+    def launch(epoch):
+        y = torch.full(shape, float("nan"), dtype=torch.float16, device=gpu)
+        _lib.check(lib.qssm_scan_forward(
+            ctypes.byref(plan), ops[0].data_ptr(), st(ops[0]), ops[1].data_ptr(), st(ops[1]), ops[2].data_ptr(), st(ops[2]),
+            ops[3].data_ptr(), st(ops[3]), y.data_ptr(), st(y), None, none, None,
+            control.data_ptr(), control.numel(), workspace.data_ptr(), workspace.numel(), epoch, stream))
+        status = ctypes.c_int32(-1)
+        _lib.check(lib.qssm_control_status(control.data_ptr(), stream, ctypes.byref(status)))
+        return y, status.value
+
+    y, status = launch(1)
+    assert status == 2 and torch.isnan(y).all()           # nothing was written
+    _lib.check(lib.qssm_zero_fill(control.data_ptr(), control.numel(), stream))
+    y, status = launch(2)
+    assert status == 0
+    _, y64 = oracle.forward_f64(x, a, b, c)
+    assert_close("y", y.cpu(), y64, TOL[torch.float16])
+
+
 def test_captured_launches_replay_with_new_inputs(gpu):
     # Forward and backward captured in one graph; every replay reads its epoch from device memory, so tiles of a
     # replay never mistake the previous replay's words for their neighbours'.  Replays alternate with eager launches
