@@ -179,13 +179,24 @@ def reset_workspaces() -> None:
         _buffers.clear()
 
 
+_plans: Dict[tuple, Plan] = {}
+
+
 def make_plan(B: int, L: int, D: int, in_dtype: torch.dtype, out_dtype: torch.dtype, direction: int,
               align_elems: int, ckpt_stride: int = 0, tune: int = 0) -> Plan:
-    plan = Plan()
-    _lib.check(
-        _lib.load().qssm_plan_scan(B, L, D, _DTYPE_CODE[in_dtype], _DTYPE_CODE[out_dtype], direction,
-                                   align_elems, ckpt_stride, tune, ctypes.byref(plan))
-    )
+    """Launch geometry for a shape (qssm_plan_scan).  Plans depend on nothing but the arguments, so they are
+    kept: small problems are bound by the host side of a launch.  Callers must not modify the result."""
+    key = (B, L, D, in_dtype, out_dtype, direction, align_elems, ckpt_stride, tune)
+    plan = _plans.get(key)
+    if plan is None:
+        plan = Plan()
+        _lib.check(
+            _lib.load().qssm_plan_scan(B, L, D, _DTYPE_CODE[in_dtype], _DTYPE_CODE[out_dtype], direction,
+                                       align_elems, ckpt_stride, tune, ctypes.byref(plan))
+        )
+        if len(_plans) >= 4096:
+            _plans.clear()
+        _plans[key] = plan
     return plan
 
 
