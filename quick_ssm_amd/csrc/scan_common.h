@@ -6,7 +6,10 @@
 // T steps x VEC columns of every operand in registers.  Lanes of one group read one contiguous
 // row piece (G * VEC * sizeof(elem) bytes; 512 B at the default geometry, which is what HBM
 // needs to stream at full rate), so all global traffic is coalesced along D while the
-// recurrence runs along L inside a lane.
+// recurrence runs along L inside a lane.  A tile that waits for its neighbours holds its operands
+// in registers, so the number of tiles a compute unit can hold bounds the bytes in flight; for
+// 16-bit storage the operands the first sweep's recurrence does not need are therefore loaded
+// straight into LDS instead (the CLDS variants of the kernels).
 //
 //   sweep 1   every lane folds its T steps into one affine map (A, X) starting from identity
 //   LDS       the NG maps of each column are exchanged; lane group j composes the maps of the
@@ -24,12 +27,14 @@
 // coherent across the XCDs' separate L2 caches.  A tile asks for its neighbours' words before
 // it issues its own operand loads and looks at the answers when they are back; in steady
 // state (tiles are claimed in time order, so neighbours ran a generation earlier) the words
-// are there and the hand-over costs no extra round trip.
+// are there and the hand-over costs no extra round trip.  Every exchanged word is HBM traffic
+// (agent-scope accesses do not stay in an XCD's L2), and the work around the words lengthens the
+// tile's stay on its compute unit: both, not the waiting, are what the hand-over costs.
 //
 // Tiles of a chain are claimed in time order through a per-chain ticket counter in a small
 // control block, so every tile a workgroup waits for was claimed by a workgroup that is already
-// running.  The control block holds nothing but the status word and the counters; the holder of
-// a chain's last ticket puts its counter back to zero.
+// running.  The control block holds the status word, a count of launches and the counters; the
+// holder of a chain's last ticket puts its counter back to zero.
 #pragma once
 
 #include <hip/hip_runtime.h>
