@@ -62,10 +62,8 @@ extern "C" {
  * `strip_cols` adjacent columns of one batch row, times `seg_len` consecutive time steps.
  * Tiles of one (batch, strip) chain are grouped in clusters of `cluster` consecutive tiles; a
  * tile reads the per-tile maps of its cluster through the workspace and one state per cluster
- * is handed from cluster to cluster.  The tiles a chain finishes with can form one larger cluster
- * (`tail` tiles): when a launch runs out of tiles, the hand-overs still to come are all that is
- * left to do, and one large cluster needs one of them where the small ones need several.
- * `ckpt_stride` is the spacing of the fp32 states h(t-1) kept for the backward.
+ * is handed from cluster to cluster.  `ckpt_stride` is the spacing of the fp32 states h(t-1)
+ * kept for the backward.
  */
 typedef struct qssm_plan {
   int32_t B, L, D;
@@ -81,11 +79,11 @@ typedef struct qssm_plan {
   int32_t n_strips;       /* ceil(D / strip_cols) */
   int32_t n_seg;          /* ceil(L / seg_len) */
   int32_t cluster;        /* tiles per cluster (power of two) */
-  int32_t n_super;        /* clusters per chain: ceil((n_seg - tail) / cluster) + (tail > 0) */
+  int32_t n_super;        /* ceil(n_seg / cluster) */
   int32_t ckpt_stride;    /* spacing (time steps) of saved states; divides seg_len */
   int32_t n_ckpt;         /* ceil(L / ckpt_stride) */
   int32_t lds_bytes;      /* dynamic LDS per workgroup */
-  int32_t tail;           /* tiles of the one larger cluster at the end of every chain (0: none); see below */
+  int32_t reserved;
   uint64_t control_bytes;   /* control block the launch needs (status word + ticket counters) */
   uint64_t workspace_bytes; /* workspace the launch needs (words exchanged between workgroups) */
   uint64_t ckpt_elems;      /* B * n_ckpt * D floats */
@@ -110,7 +108,6 @@ QSSM_API const char* qssm_error_string(void);
  *                 match one) passes the stride the saved states were written with.
  *   tune        : 0 = automatic; otherwise bit fields override single choices for sweeps, a zero field
  *                 keeping the automatic one: (g_log2 + 1) | steps << 8 | max vec << 16 |
- *                 tail code << 20 (1: no tail cluster, k >= 2: 2^(k-1) tiles) |
  *                 threads code << 24 (1: 256, 2: 512, 3: 1024) | (log2(cluster) + 1) << 28.
  * Stands in for the grid/block arithmetic of block_scan_forward_3d
  * (quick_ssm/triton_forwards.py:157-167) and block_scan_backward_3d

@@ -102,13 +102,11 @@ static int check_plan(const qssm_plan* pl, int direction) {
   if (pl->n_strips != (pl->D + pl->strip_cols - 1) / pl->strip_cols ||
       pl->n_seg != (pl->L + pl->seg_len - 1) / pl->seg_len)
     return fail(QSSM_EINVAL, "plan tile counts are inconsistent");
-  if (pl->cluster < 1 || (pl->cluster & (pl->cluster - 1)) != 0 || pl->tail < 0 || pl->tail > pl->n_seg ||
-      (pl->tail > 0 && pl->tail <= pl->cluster) ||
-      pl->n_super != (pl->n_seg - pl->tail + pl->cluster - 1) / pl->cluster + (pl->tail > 0 ? 1 : 0))
+  if (pl->cluster < 1 || (pl->cluster & (pl->cluster - 1)) != 0 ||
+      pl->n_super != (pl->n_seg + pl->cluster - 1) / pl->cluster)
     return fail(QSSM_EINVAL, "plan cluster counts are inconsistent");
-  const int widest = pl->tail > pl->cluster ? pl->tail : pl->cluster;
-  const size_t lds = direction == QSSM_FORWARD ? fwd_lds_bytes(pl->threads, pl->vec, pl->strip_cols, widest)
-                                               : bwd_lds_bytes(pl->threads, pl->vec, pl->strip_cols, widest);
+  const size_t lds = direction == QSSM_FORWARD ? fwd_lds_bytes(pl->threads, pl->vec, pl->strip_cols, pl->cluster)
+                                               : bwd_lds_bytes(pl->threads, pl->vec, pl->strip_cols, pl->cluster);
   if ((size_t)pl->lds_bytes != lds || lds > (size_t)kMaxLdsBytes)
     return fail(QSSM_EINVAL, "plan.lds_bytes=%d does not fit the geometry", pl->lds_bytes);
   // Forward lanes write a saved state only at their own first step; backward tiles read one
@@ -149,7 +147,6 @@ static void fill_geometry(Geometry* g, const qssm_plan* pl, void* control, void*
   g->seg_len = pl->seg_len;
   g->cluster = pl->cluster;
   g->n_super = pl->n_super;
-  g->tail = pl->tail;
   g->ckpt_stride = pl->ckpt_stride;
   g->n_ckpt = pl->n_ckpt;
   g->epoch = epoch;
@@ -197,7 +194,7 @@ int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int32_t ou
   // forward; the backward keeps 5 operands + h in registers, so fp32 stays at 8 bytes there.
   int vec = 4;
   if (es == 4 && direction == QSSM_BACKWARD) vec = 2;
-  const int tune_vec = (tune >> 16) & 0xf;
+  const int tune_vec = (tune >> 16) & 0xff;
   if (tune_vec == 1 || tune_vec == 2) vec = tune_vec < vec ? tune_vec : vec;
   while (vec > 1 && (align_elems % vec != 0 || (D > 0 && D % vec != 0))) vec >>= 1;
   plan->vec = vec;
@@ -303,21 +300,8 @@ int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int32_t ou
   while (cluster > 1 && lds_for(cluster) > (size_t)kMaxLdsBytes) cluster >>= 1;
   if (lds_for(cluster) > (size_t)kMaxLdsBytes) return fail(QSSM_EINVAL, "geometry needs too much LDS");
   plan->cluster = cluster;
-  // The tiles a chain finishes with form one larger cluster.  When a launch runs out of tiles, what is
-  // left is the hand-overs still to come between the tiles in flight (8 to 12 per chain on MI355X at
-  // 64 chains), one after the other; in one cluster they all need the same one state.  Forward only:
-  // the backward has no LDS left for the extra maps.  The LDS-resident c must still fit beside them.
-  int tail = 0;
-  const int tune_tail = (tune >> 20) & 0xf;
-  if (direction == QSSM_FORWARD && tune_tail != 1) {
-    tail = tune_tail >= 2 ? 1 << (tune_tail - 1) : 8;
-    while (tail > cluster &&
-           lds_for(tail) + fwd_c_lds_bytes(threads, steps) > (size_t)kMaxLdsBytes) tail >>= 1;
-    if (tail <= cluster || plan->n_seg < 2 * tail) tail = 0;
-  }
-  plan->tail = tail;
-  plan->n_super = (plan->n_seg - tail + cluster - 1) / cluster + (tail > 0 ? 1 : 0);
-  plan->lds_bytes = (int32_t)lds_for(tail > cluster ? tail : cluster);
+  plan->n_super = (plan->n_seg + cluster - 1) / cluster;
+  plan->lds_bytes = (int32_t)lds_for(cluster);
 
   const uint64_t n_chains = (uint64_t)B * plan->n_strips;
   if (n_chains * plan->n_seg > 0x7fffffffull) return fail(QSSM_EINVAL, "shape needs more than 2^31 tiles");

@@ -368,7 +368,6 @@ struct Geometry {
   int seg_len;      // time steps per tile
   int cluster;      // tiles per cluster (R, power of two)
   int n_super;      // clusters per chain
-  int tail;         // tiles of the one larger cluster every chain finishes with (0: none)
   int ckpt_stride;  // spacing of saved states
   int n_ckpt;       // saved states per (batch, column)
   unsigned epoch;   // this launch's flag value (nonzero), when the host counts launches

@@ -32,10 +32,9 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   const unsigned epoch = g.launch_count != nullptr ? *g.launch_count + 1u : g.epoch;
   float* sA = lds;                       // [NTH * VEC] per-lane map, multiplier
   float* sX = sA + NTH * VEC;            // [NTH * VEC] per-lane map, offset
-  const int slots = (g.tail > R ? g.tail : R) - 1;
-  float* sPA = sX + NTH * VEC;           // [slots * cols] maps of the earlier tiles of the cluster
-  float* sPX = sPA + slots * cols;
-  float* sH = sPX + slots * cols;        // [cols] state entering the tile
+  float* sPA = sX + NTH * VEC;           // [(R-1) * cols] maps of the earlier tiles of the cluster
+  float* sPX = sPA + (R - 1) * cols;
+  float* sH = sPX + (R - 1) * cols;      // [cols] state entering the tile
   int* sSeg = reinterpret_cast<int*>(sH + cols);
   char* sC = reinterpret_cast<char*>(sSeg) + 16;  // CLDS: [NTH / 64 waves][T rows][512 bytes] of c
 
@@ -78,14 +77,8 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
 
   // ---- ask for the neighbours' words first: they are looked at once the answers are back ------
   const bool multi = g.n_seg > 1;
-  // Clusters of R tiles, except that the chain's last `tail` tiles form one cluster of their own.
-  const int tail_start = g.n_seg - g.tail;
-  const bool in_tail = g.tail > 0 && seg >= tail_start;
-  const int s = in_tail ? g.n_super - 1 : seg / R;          // cluster of this tile
-  const int first = in_tail ? tail_start : s * R;           // its first tile
-  const int m = seg - first;                                // tiles of the cluster before this one
-  const int after = in_tail ? g.n_seg : (first + R < tail_start ? first + R : tail_start);
-  const bool cluster_last = seg == after - 1;               // this tile hands the state on
+  const int s = seg / R;               // cluster of this tile
+  const int m = seg - s * R;           // tiles of the cluster before this one
   const bool edge = (j == NG - 1);     // the last lane group holds the tile's total map
   const int lane = tid & (G - 1);      // position inside the lane group = position inside a word plane
   const unsigned long long* my_map = g.maps + ((int64_t)chain * g.n_seg + (seg - m + j)) * cols * 2 + lane;
@@ -238,7 +231,7 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
         Xt[v] = av[v] * Xp[v] + xv[v];
       }
       // Later tiles of the cluster need this tile's map; it depends on nothing, so it goes out first.
-      if (dok && !cluster_last) {
+      if (dok && m + 1 < R && seg + 1 < g.n_seg) {
         unsigned long long* mw = g.maps + ((int64_t)chain * g.n_seg + seg) * cols * 2 + lane;
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
@@ -277,7 +270,7 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
       }
     }
     if (want_state && !state_here) {
-      if (!words_wait<VEC>(prev_state, G, epoch, hin, cluster_last ? kPollChain : kPollUrgent)) raise_status(g.status, 1);
+      if (!words_wait<VEC>(prev_state, G, epoch, hin, m == R - 1 ? kPollChain : kPollUrgent)) raise_status(g.status, 1);
     }
     if (m > 0) lds_barrier();
     if (edge) {
@@ -288,7 +281,7 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
 #pragma unroll
         for (int v = 0; v < VEC; ++v) hin[v] = pa[v] * hin[v] + px[v];
       }
-      if (dok && cluster_last && seg + 1 < g.n_seg) {
+      if (dok && m == R - 1 && s + 1 < g.n_super) {
         unsigned long long* sw = g.states + ((int64_t)chain * g.n_super + s) * cols + lane;
 #pragma unroll
         for (int v = 0; v < VEC; ++v) word_publish(sw + v * G, epoch, At[v] * hin[v] + Xt[v]);

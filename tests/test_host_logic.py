@@ -49,9 +49,7 @@ def test_plans_are_consistent_and_forward_follows_backward(hip_lib, shape, dtype
             assert D % p.vec == 0 and p.vec <= align
             assert p.strip_cols == p.vec << p.g_log2
             assert p.threads in (256, 512, 1024) and p.seg_len == p.steps * (p.threads >> p.g_log2)
-            assert p.tail == 0 or (p is fwd and p.cluster < p.tail <= p.n_seg // 2)
-            assert p.n_super == -(-(p.n_seg - p.tail) // p.cluster) + (1 if p.tail else 0)
-            assert 0 < p.lds_bytes <= 64 * 1024
+            assert p.n_super == -(-p.n_seg // p.cluster) and 0 < p.lds_bytes <= 64 * 1024
             assert p.n_strips * p.strip_cols >= D > (p.n_strips - 1) * p.strip_cols
             assert p.n_seg * p.seg_len >= L > (p.n_seg - 1) * p.seg_len
             assert p.seg_len % p.ckpt_stride == 0
@@ -184,9 +182,7 @@ def _tile_accesses(plan, B, L, D):
             if plan.n_seg > 1:
                 edge = dl[dok]
                 hi_word = max(hi_word, maps_off + int((((chain * plan.n_seg + seg) * cols + edge) * 2).max() + 2 * plan.vec) * 8)
-                tail_start = plan.n_seg - plan.tail
-                s = plan.n_super - 1 if plan.tail and seg >= tail_start else seg // plan.cluster
-                assert 0 <= s < plan.n_super
+                s = seg // plan.cluster
                 hi_word = max(hi_word, states_off + int(((chain * plan.n_super + s) * cols + edge).max() + plan.vec) * 8)
     assert NG * plan.steps == plan.seg_len
     return lo_elem, hi_elem, hi_ckpt, hi_word
