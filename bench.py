@@ -71,12 +71,17 @@ def cpu_baseline(torch, workload, shape, dtype, out_dtype, a_lo, a_span):
 
     B, L, D = shape
     # One batch row with every column of the workload.  The reference's backward through its in-place slice writes
-    # costs O(L^2) whole-row copies, so rows are cut to 2048 steps: 10-20 s on the hosts of this pool.
+    # costs O(L^2) whole-row copies once a row outgrows the host's caches, so rows are cut to 2048 steps.
     sB, sL, sD = 1, min(L, 2048), D
     ops, _ = make_operands(torch, (sB, sL, sD), dtype, out_dtype, a_lo, a_span, "cpu")
-    t0 = time.perf_counter()
-    reference_scan_with_grads(*ops, out_dtype=out_dtype)
-    dt = time.perf_counter() - t0
+    # Hosts differ by more than 10x on this path: repeat the row until about 10 s of CPU work are on the clock.
+    rows, dt = 0, 0.0
+    while dt < 10.0 and rows < 64:
+        t0 = time.perf_counter()
+        reference_scan_with_grads(*ops, out_dtype=out_dtype)
+        dt += time.perf_counter() - t0
+        rows += 1
+    sB = rows
     n = sB * sL * sD
     es, os_ = ops[0].element_size(), ops[4].element_size()
     nbytes = n * (8 * es + 2 * os_)
@@ -86,7 +91,7 @@ def cpu_baseline(torch, workload, shape, dtype, out_dtype, a_lo, a_span):
         "cores": torch.get_num_threads(),
         "kind": "port",
         "sample": f"reference CPU path (python loop over batch and time, torch autograd backward) fwd+bwd on a "
-                  f"slice B={sB} L={sL} D={sD} of {workload}, {dt:.2f} s, host cpu_count={os.cpu_count()}",
+                  f"slice L={sL} D={sD} of {workload} run {sB} time(s), {dt:.2f} s, host cpu_count={os.cpu_count()}",
         "melem_per_s": n / dt / 1e6,
         "seconds": dt,
     }
