@@ -276,6 +276,31 @@ QSSM_API int qssm_gates_backward(const void* g_a, const void* g_x, const void* g
                         int64_t rows, int32_t S, int32_t in_dtype, int32_t out_dtype, void* stream);
 
 /*
+ * RMSNorm of the SSM layer over the last axis: y = x * weight / sqrt(mean(x^2) + eps).
+ * x is [rows, H] with row stride ld_x elements, weight [H], y [rows, H] contiguous, all stored as `dtype`
+ * (f32, f16 or bf16); fp32 arithmetic, one rounding per result.  `rstd` ([rows] fp32, or NULL) receives
+ * 1 / sqrt(mean(x^2) + eps) per row for the backward.  One pass: x is read once, y written once.
+ * Replaces RMSNorm.forward, quick_ssm/layers.py:14-17 (pow, mean, add, sqrt, divide, multiply as six
+ * passes).
+ */
+QSSM_API int qssm_rmsnorm_forward(const void* x, int64_t ld_x, const void* weight, void* y, float* rstd,
+                         int64_t rows, int32_t H, float eps, int32_t dtype, void* stream);
+
+/*
+ * Backward of the RMSNorm in one pass over dy and x (row strides ld_dy, ld_x elements):
+ *   g = dy * weight, s = sum(g * x), r = rstd:  dx = r * g - x * r^3 * s / H,  dweight = sum over rows dy * x * r.
+ * dx is [rows, H] contiguous and dweight [H], both stored as `dtype`.  `rstd` may be NULL (r is then
+ * recomputed from x and eps).  `partial` is fp32 scratch of `partial_rows` x H floats
+ * (partial_rows >= QSSM_RMSNORM_MIN_PARTIAL_ROWS; more rows, up to 512, let more workgroups run); dweight
+ * is summed from it in a fixed order by a second small launch, so results repeat bit for bit.
+ * Replaces what autograd records for quick_ssm/layers.py:14-17.
+ */
+#define QSSM_RMSNORM_MIN_PARTIAL_ROWS 8
+QSSM_API int qssm_rmsnorm_backward(const void* dy, int64_t ld_dy, const void* x, int64_t ld_x, const void* weight,
+                          const float* rstd, void* dx, void* dweight, float* partial, int32_t partial_rows,
+                          int64_t rows, int32_t H, float eps, int32_t dtype, void* stream);
+
+/*
  * Streaming copy of `bytes` bytes (16-byte aligned, multiple of 16) on `stream`.  Not part of
  * the scan: it is the known-size kernel against which rocprof's FETCH_SIZE / WRITE_SIZE
  * counters and the achievable-bandwidth ceiling are calibrated by the benchmark.

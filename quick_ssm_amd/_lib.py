@@ -16,6 +16,7 @@ LIB_PATH = Path(__file__).resolve().parent / LIB_NAME
 
 QSSM_F32, QSSM_F16, QSSM_BF16 = 0, 1, 2
 QSSM_FORWARD, QSSM_BACKWARD = 0, 1
+QSSM_RMSNORM_MIN_PARTIAL_ROWS = 8
 QSSM_EINVAL, QSSM_EALIGN, QSSM_EWORKSPACE, QSSM_ESTATE = -1, -2, -3, -4
 
 EXPORTED_SYMBOLS = (
@@ -30,6 +31,8 @@ EXPORTED_SYMBOLS = (
     "qssm_scan_backward_carry",
     "qssm_gates_forward",
     "qssm_gates_backward",
+    "qssm_rmsnorm_forward",
+    "qssm_rmsnorm_backward",
     "qssm_copy_bytes",
 )
 
@@ -117,6 +120,10 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.qssm_gates_forward.argtypes = [vp, i64] * 5 + [vp] * 4 + [i64, i32, i32, i32, vp]
     lib.qssm_gates_backward.restype = ctypes.c_int
     lib.qssm_gates_backward.argtypes = [vp] * 4 + [vp, i64] * 4 + [vp] * 5 + [i64, i32, i32, i32, vp]
+    lib.qssm_rmsnorm_forward.restype = ctypes.c_int
+    lib.qssm_rmsnorm_forward.argtypes = [vp, i64, vp, vp, vp, i64, i32, ctypes.c_float, i32, vp]
+    lib.qssm_rmsnorm_backward.restype = ctypes.c_int
+    lib.qssm_rmsnorm_backward.argtypes = [vp, i64, vp, i64, vp, vp, vp, vp, vp, i32, i64, i32, ctypes.c_float, i32, vp]
     lib.qssm_copy_bytes.restype = ctypes.c_int
     lib.qssm_copy_bytes.argtypes = [vp, vp, u64, vp]
 

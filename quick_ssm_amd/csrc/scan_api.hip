@@ -529,6 +529,44 @@ int qssm_gates_backward(const void* g_a, const void* g_x, const void* g_c, const
   return e == hipSuccess ? 0 : hip_fail(e, "gates_bwd_kernel launch");
 }
 
+int qssm_rmsnorm_forward(const void* x, int64_t ld_x, const void* weight, void* y, float* rstd, int64_t rows,
+                         int32_t H, float eps, int32_t dtype, void* stream) {
+  const int es = dtype_size(dtype);
+  if (es == 0) return fail(QSSM_EINVAL, "unknown dtype code");
+  if (rows < 0 || H < 0) return fail(QSSM_EINVAL, "negative dimension");
+  if (rows == 0 || H == 0) return 0;
+  if (!x || !weight || !y) return fail(QSSM_EINVAL, "NULL tensor");
+  if (ld_x < H) return fail(QSSM_EINVAL, "row stride below H");
+  if ((int64_t)H * es > 0x7fffffffll) return fail(QSSM_EINVAL, "row too wide");
+  NormFwdArgs args{x, ld_x, weight, y, rstd, rows, H, eps};
+  const int vec = gate_vec(H, {{x, ld_x}, {weight, H}, {y, H}}, es, {}, es);
+  if (!launch_norm_any(dtype, &args, nullptr, vec, 0, nullptr, (hipStream_t)stream))
+    return fail(QSSM_EINVAL, "rmsnorm storage type %d is not built", dtype);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : hip_fail(e, "rmsnorm_fwd_kernel launch");
+}
+
+int qssm_rmsnorm_backward(const void* dy, int64_t ld_dy, const void* x, int64_t ld_x, const void* weight,
+                          const float* rstd, void* dx, void* dweight, float* partial, int32_t partial_rows,
+                          int64_t rows, int32_t H, float eps, int32_t dtype, void* stream) {
+  const int es = dtype_size(dtype);
+  if (es == 0) return fail(QSSM_EINVAL, "unknown dtype code");
+  if (rows < 0 || H < 0) return fail(QSSM_EINVAL, "negative dimension");
+  if (H == 0) return 0;
+  if (!dweight || !partial) return fail(QSSM_EINVAL, "NULL tensor");
+  if (rows > 0 && (!dy || !x || !weight || !dx)) return fail(QSSM_EINVAL, "NULL tensor");
+  if (ld_dy < H || ld_x < H) return fail(QSSM_EINVAL, "row stride below H");
+  if ((int64_t)H * es > 0x7fffffffll) return fail(QSSM_EINVAL, "row too wide");
+  if (partial_rows < QSSM_RMSNORM_MIN_PARTIAL_ROWS)
+    return fail(QSSM_EINVAL, "partial needs at least %d rows of H floats", QSSM_RMSNORM_MIN_PARTIAL_ROWS);
+  NormBwdArgs args{dy, ld_dy, x, ld_x, weight, rstd, dx, partial, rows, H, eps};
+  const int vec = rows == 0 ? 1 : gate_vec(H, {{dy, ld_dy}, {x, ld_x}, {weight, H}, {dx, H}}, es, {}, es);
+  if (!launch_norm_any(dtype, nullptr, &args, vec, partial_rows, dweight, (hipStream_t)stream))
+    return fail(QSSM_EINVAL, "rmsnorm storage type %d is not built", dtype);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : hip_fail(e, "rmsnorm_bwd_kernel launch");
+}
+
 int qssm_copy_bytes(void* dst, const void* src, uint64_t bytes, void* stream) {
   if (bytes == 0) return 0;
   if (dst == nullptr || src == nullptr) return fail(QSSM_EINVAL, "NULL argument");

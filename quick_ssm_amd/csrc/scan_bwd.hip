@@ -96,10 +96,8 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   const int cnt = last - seg;                                // tiles of the cluster after this one
   const bool edge = (j == 0);  // the first lane group holds the tile's total reverse map
   const int lane = tid & (G - 1);  // position inside the lane group = position inside a word plane
-  const unsigned long long* my_map = g.maps + ((int64_t)chain * g.n_seg + (seg + 1 + j)) * cols * 2 + lane;
   const unsigned long long* next_state = g.states + ((int64_t)chain * g.n_super + (s + 1)) * cols + lane;
-  const bool want_map = multi && dok && j < cnt;                       // this lane group fetches the map of tile (seg + 1 + j)
-  const bool want_state = multi && dok && edge && s + 1 < g.n_super;   // and the first group the next cluster's carry
+  const bool want_state = multi && dok && edge && s + 1 < g.n_super;   // the first group fetches the next cluster's carry
   Peek<VEC> pk_state;
   pk_state.clear();
   if (want_state) pk_state.issue(next_state, G);

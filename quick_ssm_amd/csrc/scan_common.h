@@ -448,4 +448,36 @@ struct GateBwdArgs {
 bool launch_gates_any(int in_dtype, int out_dtype, const GateFwdArgs* f, const GateBwdArgs* b, int vec,
                       hipStream_t stream);
 
+// ---- RMSNorm of the SSM layer (rmsnorm.hip) ----------------------------------------------------------
+
+struct NormFwdArgs {
+  const void* x;      // [rows, H], row stride ld_x elements
+  int64_t ld_x;
+  const void* w;      // [H]
+  void* y;            // [rows, H] contiguous
+  float* rstd;        // [rows] 1 / sqrt(mean(x^2) + eps), or null
+  int64_t rows;
+  int H;
+  float eps;
+};
+
+struct NormBwdArgs {
+  const void* dy;     // [rows, H], row stride ld_dy elements
+  int64_t ld_dy;
+  const void* x;      // [rows, H], row stride ld_x elements
+  int64_t ld_x;
+  const void* w;      // [H]
+  const float* rstd;  // [rows] as the forward stored it, or null (recomputed from x and eps)
+  void* dx;           // [rows, H] contiguous
+  float* partial;     // [partial rows, H] fp32 scratch for dw
+  int64_t rows;
+  int H;
+  float eps;
+};
+
+// Exactly one of f, b is non-null; dw and max_partial_rows belong to the backward.  False if the
+// storage type or vec is not built, or `partial` is too small for one launch.
+bool launch_norm_any(int dtype, const NormFwdArgs* f, const NormBwdArgs* b, int vec, int max_partial_rows, void* dw,
+                     hipStream_t stream);
+
 }  // namespace qssm

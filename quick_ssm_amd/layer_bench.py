@@ -1,0 +1,160 @@
+"""Times the SSM layer's HIP passes around the scan, and the layer step they sit in, on one GPU.
+
+    python -m quick_ssm_amd.layer_bench [--batch 16] [--length 2048] [--hidden 1024] [--mult 4.0]
+                                        [--param-dtype float32] [--compute-dtype float16] [--steps 20] [--warmup 5]
+
+Defaults are the layer configuration of the reference's example scripts (quick_ssm/example_layer.py,
+copy_train.py:26: state = 4 x hidden, fp32 parameters, fp16 scan operands).  Each pass is timed alone
+through the C ABI with HIP events on the launch stream, and priced against HBM (8 TB/s) with its
+algorithmic bytes: what it must read and write once.
+
+    rmsnorm forward   rows x H x (s + s)            x in, y out
+    rmsnorm backward  rows x H x (2 s + s)          dy, x in, dx out
+    gates forward     rows x S x (5 s_p + 4 s_c)    five projections in, four operands out
+    gates backward    rows x S x (4 s_c + 4 s_p + 5 s_p)
+    scan forward      rows x S x (4 s_c + s_y)      scan backward  rows x S x (8 s_c + s_y)
+
+One JSON line is printed; `layer_step_ms` is forward + backward of the whole layer (GEMMs included)
+through autograd, with the fused passes and, beside it, with the same formulas as separate torch ops.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+
+HBM_PEAK_GBS = 8000.0
+
+
+def _time_us(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps * 1e3
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--length", type=int, default=2048)
+    ap.add_argument("--hidden", type=int, default=1024)
+    ap.add_argument("--mult", type=float, default=4.0)
+    ap.add_argument("--param-dtype", default="float32")
+    ap.add_argument("--compute-dtype", default="float16")
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    args = ap.parse_args()
+
+    import torch
+
+    from . import _lib, gates, hip_scan, layers, norm
+
+    if not torch.cuda.is_available():
+        print("layer_bench needs a GPU", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    torch.manual_seed(0)
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    pdt, cdt = getattr(torch, args.param_dtype), getattr(torch, args.compute_dtype)
+    B, L, H = args.batch, args.length, args.hidden
+    S = int(H * args.mult)
+    rows = B * L
+    sp, sc = torch.empty(0, dtype=pdt).element_size(), torch.empty(0, dtype=cdt).element_size()
+    code = {torch.float32: _lib.QSSM_F32, torch.float16: _lib.QSSM_F16, torch.bfloat16: _lib.QSSM_BF16}
+    passes = {}
+
+    def record(name, us, nbytes):
+        passes[name] = {"us": us, "algorithmic_bytes": nbytes, "gbs": nbytes / us / 1e3,
+                        "frac_of_hbm_peak": nbytes / us / 1e3 / HBM_PEAK_GBS}
+
+    # ---- RMSNorm ------------------------------------------------------------------------------------
+    x = torch.randn(rows, H, device=dev).to(pdt)
+    w = (torch.rand(H, device=dev) + 0.5).to(pdt)
+    dy = torch.randn(rows, H, device=dev).to(pdt)
+    y, dx, dw = torch.empty_like(x), torch.empty_like(x), torch.empty_like(w)
+    rstd = torch.empty(rows, device=dev)
+    partial = torch.empty(norm.PARTIAL_ROWS, H, device=dev)
+    us = _time_us(torch, lambda: _lib.check(lib.qssm_rmsnorm_forward(
+        x.data_ptr(), H, w.data_ptr(), y.data_ptr(), rstd.data_ptr(), rows, H, 1e-5, code[pdt], stream)),
+        args.steps, args.warmup)
+    record("rmsnorm_forward", us, rows * H * 2 * sp)
+    us = _time_us(torch, lambda: _lib.check(lib.qssm_rmsnorm_backward(
+        dy.data_ptr(), H, x.data_ptr(), H, w.data_ptr(), rstd.data_ptr(), dx.data_ptr(), dw.data_ptr(),
+        partial.data_ptr(), norm.PARTIAL_ROWS, rows, H, 1e-5, code[pdt], stream)), args.steps, args.warmup)
+    record("rmsnorm_backward", us, rows * H * 3 * sp)
+    del x, y, dy, dx
+
+    # ---- gate prologue ------------------------------------------------------------------------------
+    if (pdt, cdt) in gates._BUILT:
+        z = [torch.randn(rows, S, device=dev).to(pdt) for _ in range(5)]
+        ops = [torch.empty(rows, S, dtype=cdt, device=dev) for _ in range(4)]
+        g = [torch.randn(rows, S, device=dev).to(cdt) for _ in range(4)]
+        dz = [torch.empty(rows, S, dtype=pdt, device=dev) for _ in range(5)]
+        fargs = []
+        for t in z:
+            fargs += [t.data_ptr(), S]
+        us = _time_us(torch, lambda: _lib.check(lib.qssm_gates_forward(
+            *fargs, *[o.data_ptr() for o in ops], rows, S, code[pdt], code[cdt], stream)), args.steps, args.warmup)
+        record("gates_forward", us, rows * S * (5 * sp + 4 * sc))
+        bargs = [t.data_ptr() for t in g]
+        for t in (z[0], z[2], z[3], z[4]):
+            bargs += [t.data_ptr(), S]
+        us = _time_us(torch, lambda: _lib.check(lib.qssm_gates_backward(
+            *bargs, *[o.data_ptr() for o in dz], rows, S, code[pdt], code[cdt], stream)), args.steps, args.warmup)
+        record("gates_backward", us, rows * S * (4 * sc + 9 * sp))
+        del z, g, dz
+
+        # ---- the scan on operands of that shape (y and dy in the parameters' storage) -----------------
+        a, xs, c, b = ops
+        a.uniform_(0.9, 1.0)
+        xs.normal_()
+        c.uniform_(0.0, 1.0)
+        b.normal_(0.0, 0.1)
+        a3, x3, c3, b3 = (t.view(B, L, S) for t in (a, xs, c, b))
+        gy = torch.randn(B, L, S, device=dev).to(pdt)
+        with torch.no_grad():
+            _, _, ckpt, stride = hip_scan.scan_forward(x3, a3, b3, c3, out_dtype=pdt)
+            us = _time_us(torch, lambda: hip_scan.scan_forward(x3, a3, b3, c3, out_dtype=pdt), args.steps, args.warmup)
+            record("scan_forward", us, rows * S * (4 * sc + sp))
+            us = _time_us(torch, lambda: hip_scan.scan_backward(x3, a3, b3, c3, gy, ckpt=ckpt, ckpt_stride=stride),
+                          args.steps, args.warmup)
+            record("scan_backward", us, rows * S * (8 * sc + sp))
+        del ops, gy, ckpt
+
+    # ---- the whole layer step, fused passes against separate torch ops ---------------------------------
+    layer = layers.SSM(H, args.mult, dtype=pdt, device=dev, compute_dtype=cdt)
+    inp = torch.randn(B, L, H, device=dev).to(pdt).requires_grad_(True)
+
+    def step():
+        inp.grad = None
+        layer.zero_grad(set_to_none=True)
+        layer(inp).sum().backward()
+
+    fused_ms = _time_us(torch, step, max(3, args.steps // 2), 2) / 1e3
+    keep = layers.gate_prologue, layers.rms_norm
+    layers.gate_prologue, layers.rms_norm = gates.gates_reference, norm.rms_norm_reference
+    try:
+        torch_ms = _time_us(torch, step, max(3, args.steps // 2), 2) / 1e3
+    finally:
+        layers.gate_prologue, layers.rms_norm = keep
+
+    print(json.dumps({
+        "config": {"batch": B, "length": L, "hidden": H, "state": S, "param_dtype": args.param_dtype,
+                   "compute_dtype": args.compute_dtype},
+        "passes": passes,
+        "layer_step_ms": {"fused_passes": fused_ms, "torch_ops_for_norm_and_gates": torch_ms},
+        "workspace_status": hip_scan.workspace_status(),
+    }), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

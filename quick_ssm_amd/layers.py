@@ -3,7 +3,7 @@
 Same constructor arguments, parameter names (so state dicts interchange) and forward keywords as
 the reference's quick_ssm/layers.py:9-107.  The projections stay on torch GEMMs; the gate
 activations and casts between them and the scan are one fused HIP pass (quick_ssm_amd/gates.py),
-and the scan is the HIP path.  Roles of the projections
+the pre-norm is one fused HIP pass each way (quick_ssm_amd/norm.py), and the scan is the HIP path.  Roles of the projections
 (quick_ssm/test_swiglu_equiv.py:60-70): A_proj -> forget gate a, B_proj -> the scan's input x,
 D_proj -> input gate b, C_proj_a/C_proj_b -> SwiGLU output gate c, out_proj -> output.
 """
@@ -15,6 +15,7 @@ import torch
 import torch.nn as nn
 
 from .gates import gate_prologue
+from .norm import rms_norm
 from .scan_interface import scan
 
 
@@ -27,8 +28,7 @@ class RMSNorm(nn.Module):
         self.weight = nn.Parameter(torch.ones(hidden_size, dtype=dtype, device=device))
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        rms = torch.sqrt(x.pow(2).mean(dim=-1, keepdim=True) + self.eps)
-        return x * (self.weight / rms)
+        return rms_norm(x, self.weight, self.eps)
 
 
 class SSM(nn.Module):

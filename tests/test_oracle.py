@@ -214,6 +214,47 @@ def test_gate_oracle_against_torch_library_routines_and_differences():
     assert np.all(np.isfinite(sat[0])) and sat[0][0, 0] == 0.0 and sat[0][0, 1] == 1.0 and sat[2][0, 0] == 0.0
 
 
+def test_rmsnorm_oracle_against_torch_library_routine_and_differences():
+    # Pins oracle/rmsnorm_oracle.py: forward against torch.nn.functional.rms_norm in float64, backward against
+    # torch's autograd of that library routine, against central differences, and through what the formula fixes.
+    from oracle import rmsnorm_oracle
+    import torch.nn.functional as F
+    gen = torch.Generator().manual_seed(23)
+    x = (torch.randn(3, 5, 11, generator=gen, dtype=torch.float64) * 2).requires_grad_(True)
+    w = (torch.rand(11, generator=gen, dtype=torch.float64) + 0.5).requires_grad_(True)
+    dy = torch.randn(3, 5, 11, generator=gen, dtype=torch.float64)
+    eps = 1e-5
+    y = F.rms_norm(x, (11,), w, eps)
+    np.testing.assert_allclose(rmsnorm_oracle.rmsnorm_forward_f64(x, w, eps), y.detach().numpy(), rtol=1e-14)
+    (y * dy).sum().backward()
+    dx, dw = rmsnorm_oracle.rmsnorm_backward_f64(dy, x, w, eps)
+    np.testing.assert_allclose(dx, x.grad.numpy(), rtol=1e-11, atol=1e-14)
+    np.testing.assert_allclose(dw, w.grad.numpy(), rtol=1e-11, atol=1e-14)
+    # central differences on one element of x and of the weight
+    xs, ws, gs = x.detach().numpy().copy(), w.detach().numpy().copy(), dy.numpy()
+
+    def loss(xv, wv):
+        return float((rmsnorm_oracle.rmsnorm_forward_f64(xv, wv, eps) * gs).sum())
+
+    hi, lo = xs.copy(), xs.copy()
+    hi[1, 2, 3] += 1e-6
+    lo[1, 2, 3] -= 1e-6
+    fd = (loss(hi, ws) - loss(lo, ws)) / 2e-6
+    assert abs(fd - dx[1, 2, 3]) <= 1e-7 * max(1.0, abs(fd))
+    hi, lo = ws.copy(), ws.copy()
+    hi[4] += 1e-6
+    lo[4] -= 1e-6
+    fd = (loss(xs, hi) - loss(xs, lo)) / 2e-6
+    assert abs(fd - dw[4]) <= 1e-7 * max(1.0, abs(fd))
+    # eps = 0: y does not change when x is scaled, every row of y / w has unit mean square, and dx is
+    # orthogonal to x (the loss cannot change along the direction that only rescales the row)
+    y0 = rmsnorm_oracle.rmsnorm_forward_f64(xs, ws, 0.0)
+    np.testing.assert_allclose(rmsnorm_oracle.rmsnorm_forward_f64(7.5 * xs, ws, 0.0), y0, rtol=1e-13)
+    np.testing.assert_allclose(np.mean((y0 / ws) ** 2, axis=-1), 1.0, rtol=1e-13)
+    dx0, _ = rmsnorm_oracle.rmsnorm_backward_f64(gs, xs, ws, 0.0)
+    assert np.max(np.abs(np.sum(dx0 * xs, axis=-1))) <= 1e-12 * np.max(np.abs(dx0)) * np.max(np.abs(xs)) * 11
+
+
 def test_c_and_torch_flavours_agree_bitwise_in_fp32():
     x, a, b, c, dy = make_inputs((2, 130, 5), seed=3)
     h_c = oracle.forward_f32_seq(x, a, b)
