@@ -95,12 +95,13 @@ def _align_elems(tensors: Sequence[Optional[Tensor]], D: int) -> int:
     return 1
 
 
-_device_counted = threading.local()
+_device_counted_depth = 0  # contexts open right now, in any thread (guarded by _ws_lock)
 
 
 class device_counted_launches:
-    """Context manager: scan launches inside number themselves in their control block (epoch argument 0), as
-    launches recorded into a graph do, and use the buffers kept for such launches.
+    """Context manager: scan launches made while it is open, from any thread (autograd runs the backward on its
+    own), number themselves in their control block (epoch argument 0), as launches recorded into a graph do, and use
+    the buffers kept for such launches.
 
     Launches being recorded into a graph do this by themselves, but cannot allocate: run the work once inside this
     context, on the stream that will capture, and the control block and workspace exist (large enough) when the
@@ -108,12 +109,15 @@ class device_counted_launches:
     """
 
     def __enter__(self):
-        self._old = getattr(_device_counted, "on", False)
-        _device_counted.on = True
+        global _device_counted_depth
+        with _ws_lock:
+            _device_counted_depth += 1
         return self
 
     def __exit__(self, *exc):
-        _device_counted.on = self._old
+        global _device_counted_depth
+        with _ws_lock:
+            _device_counted_depth -= 1
         return False
 
 
@@ -130,7 +134,7 @@ def _launch_buffers(device: torch.device, stream: int, plan: Plan) -> Tuple[Tens
     whose 32-bit host numbering is used up, is replaced by a fresh zeroed one.
     """
     capturing = bool(torch.cuda.is_current_stream_capturing())
-    on_device = capturing or getattr(_device_counted, "on", False)
+    on_device = capturing or _device_counted_depth > 0
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream, on_device)
     with _ws_lock:
         buf = _buffers.get(key)
