@@ -300,7 +300,10 @@ static bool launch_norm(const NormFwdArgs* f, const NormBwdArgs* b, int vec, int
   const int rows_per_wg = wide ? 1 : kNormWaves / W;
   int64_t blocks = (rows + rows_per_wg - 1) / rows_per_wg;
   if (blocks < 1) blocks = 1;
+  // Forward: one short workgroup per pass over rows_per_wg rows, started in index order.  Backward: at most
+  // 512 workgroups that stay (each sums its own dweight) and stride through the rows together.
   int grid = (int)(blocks < 512 ? blocks : 512);
+  if (f) grid = (int)(blocks < (1 << 30) ? blocks : (1 << 30));
   if (b && grid > max_partial_rows) grid = max_partial_rows;
   if (grid < 1) return false;
   bool done = false;

@@ -59,19 +59,24 @@ __global__ void __launch_bounds__(256) fill_zero_kernel(uint4* p, uint64_t n16) 
   for (; i < n16; i += stride) p[i] = make_uint4(0, 0, 0, 0);
 }
 
-// Grid-stride 16-byte copy: the calibration kernel of known traffic (bytes read = bytes written).
+// 16-byte copy, the calibration kernel of known traffic (bytes read = bytes written): one workgroup per
+// 16 KiB, started in index order and gone after one step, so that the resident workgroups cover one
+// narrow window of both buffers (workgroups that stay and stride through the buffers copy a fifth slower).
 __global__ void __launch_bounds__(256) copy_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src,
                                                    uint64_t n16) {
-  uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
-  for (; i + 3 * stride < n16; i += 4 * stride) {
-    const uint4 v0 = src[i], v1 = src[i + stride], v2 = src[i + 2 * stride], v3 = src[i + 3 * stride];
-    dst[i] = v0;
-    dst[i + stride] = v1;
-    dst[i + 2 * stride] = v2;
-    dst[i + 3 * stride] = v3;
+  for (uint64_t base = (uint64_t)blockIdx.x * 1024u; base < n16; base += (uint64_t)gridDim.x * 1024u) {
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    const u32x4* s = reinterpret_cast<const u32x4*>(src);
+    u32x4* d = reinterpret_cast<u32x4*>(dst);
+    const uint64_t i = base + threadIdx.x;
+    u32x4 v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if (i + 256u * k < n16) v[k] = __builtin_nontemporal_load(s + i + 256u * k);
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if (i + 256u * k < n16) __builtin_nontemporal_store(v[k], d + i + 256u * k);
   }
-  for (; i < n16; i += stride) dst[i] = src[i];
 }
 
 static bool aligned_to(const void* p, int64_t sb, int64_t sl, int elem_bytes, int vec) {
@@ -573,8 +578,8 @@ int qssm_copy_bytes(void* dst, const void* src, uint64_t bytes, void* stream) {
   if (((uintptr_t)dst) % 16 != 0 || ((uintptr_t)src) % 16 != 0 || bytes % 16 != 0)
     return fail(QSSM_EALIGN, "copy needs 16-byte alignment and a multiple of 16 bytes");
   const uint64_t n16 = bytes / 16;
-  uint64_t blocks = (n16 + 256 * 4 - 1) / (256 * 4);
-  if (blocks > 256 * 32) blocks = 256 * 32;
+  uint64_t blocks = (n16 + 1023) / 1024;
+  if (blocks > (1u << 30)) blocks = 1u << 30;
   if (blocks == 0) blocks = 1;
   hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (uint4*)dst,
                      (const uint4*)src, n16);

@@ -598,3 +598,16 @@ def test_config3_ssm_layer_matches_sequential_path(gpu):
     assert_close("layer dx", dx_gpu, dx_ref.double().numpy(), 1e-2)
     for n in g_ref:
         assert_close(f"grad {n}", g_gpu[n], g_ref[n].double().numpy(), 2e-2)
+
+
+def test_calibration_copy_moves_every_byte(gpu):
+    # qssm_copy_bytes is the kernel of known traffic that the HBM counters are scaled by: sizes that are not a
+    # multiple of a workgroup's 16 KiB, one 16-byte piece, nothing
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(gpu).cuda_stream
+    for nbytes in (16, 16 * 1023, 16 * 1024, 16 * 1025, (3 << 20) + 48):
+        src = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device=gpu)
+        dst = torch.zeros(nbytes + 16, dtype=torch.uint8, device=gpu)
+        assert lib.qssm_copy_bytes(dst.data_ptr(), src.data_ptr(), nbytes, stream) == 0
+        assert torch.equal(dst[:nbytes], src) and int(dst[nbytes:].sum()) == 0
+    assert lib.qssm_copy_bytes(None, None, 0, stream) == 0
