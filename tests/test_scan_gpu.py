@@ -319,7 +319,7 @@ def test_carried_state_argument_errors_and_empty_piece(gpu):
 # ---- launch numbering: by the caller, by the library, and under graph replay --------------------------------
 
 def test_c_abi_with_caller_counted_epochs(gpu):
-    # the raw C ABI the way INTEGRATION.md shows it: own control block and workspace, epochs 1, 2, 3 from the caller
+    # the raw C ABI as a caller outside this package would use it: own control block and workspace, epochs 1, 2, 3 from the caller
     import ctypes
     lib = _lib.load()
     shape = (2, 900, 256)
