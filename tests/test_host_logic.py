@@ -200,3 +200,36 @@ def test_tile_index_arithmetic_stays_in_bounds(hip_lib, shape, dtype):
             assert lo >= 0 and hi == B * L * D - 1          # every element is covered, nothing beyond
             assert hi_ckpt < plan.ckpt_elems
             assert hi_word <= plan.workspace_bytes
+
+
+def test_plan_invariants_over_random_shapes(hip_lib):
+    # a seeded sweep over shapes, alignments, storage pairs and directions: whatever the planner picks must describe
+    # a launch the kernels can run (lane counts, tile lengths, LDS, buffer sizes), for the backward first and then for
+    # a forward that saves the states that backward will read
+    import random
+    rng = random.Random(1234)
+    pairs = [(torch.float32, torch.float32), (torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16),
+             (torch.float16, torch.float32), (torch.bfloat16, torch.float32)]
+    for _ in range(400):
+        B = rng.choice([1, 1, 2, 3, 8, 17, 64])
+        L = rng.choice([1, 2, 7, 31, 32, 33, 64, 100, 255, 256, 1000, 4096, 5000, 65536, 100001])
+        D = rng.choice([1, 2, 3, 4, 6, 8, 12, 60, 64, 100, 256, 260, 1024, 2048, 4100])
+        dt, odt = rng.choice(pairs)
+        align = rng.choice([1, 2, 4, 8])
+        bwd = hip_scan.make_plan(B, L, D, dt, odt, _lib.QSSM_BACKWARD, align)
+        fwd = hip_scan.make_plan(B, L, D, dt, odt, _lib.QSSM_FORWARD, align, bwd.seg_len)
+        for p in (bwd, fwd):
+            what = (B, L, D, dt, odt, align, p.describe())
+            assert p.vec in (1, 2, 4) and D % p.vec == 0 and align % p.vec == 0, what
+            assert p.steps in (4, 8) and p.threads in (256, 512, 1024), what
+            assert 1 <= (1 << p.g_log2) <= p.threads and p.strip_cols == p.vec << p.g_log2, what
+            assert p.seg_len == p.steps * (p.threads >> p.g_log2) and p.seg_len % p.ckpt_stride == 0, what
+            assert p.n_strips == -(-D // p.strip_cols) and p.n_seg == -(-L // p.seg_len), what
+            assert p.cluster in (1, 2, 4, 8) and p.n_super == -(-p.n_seg // p.cluster), what
+            assert 0 < p.lds_bytes <= 64 * 1024, what
+            chains = B * p.n_strips
+            assert p.control_bytes >= 64 + 64 * chains and p.control_bytes % 256 == 0, what
+            words = chains * (p.n_seg * 2 + p.n_super) * p.strip_cols * 8
+            assert (p.workspace_bytes >= words if p.n_seg > 1 else p.workspace_bytes == 0), what
+            assert p.ckpt_elems == B * p.n_ckpt * D and p.n_ckpt == -(-L // p.ckpt_stride), what
+        assert fwd.ckpt_stride == bwd.ckpt_stride == bwd.seg_len
