@@ -103,9 +103,10 @@ class _HipScanFunction(torch.autograd.Function):
         if not checkpoint and not whole:
             h_saved = torch.empty(x.shape, dtype=torch.float32, device=x.device)
         for bs_, ds_ in tiles:
+            # the common case, one launch over the whole tensor, skips four view constructions
+            ops = (xs, as_, bs, cs) if whole else tuple(t[bs_, :, ds_] for t in (xs, as_, bs, cs))
             yt, ht, ckpt, stride = hip_scan.scan_forward(
-                xs[bs_, :, ds_], as_[bs_, :, ds_], bs[bs_, :, ds_], cs[bs_, :, ds_],
-                out_dtype=k_out, want_h=not checkpoint, want_ckpt=bool(checkpoint),
+                *ops, out_dtype=k_out, want_h=not checkpoint, want_ckpt=bool(checkpoint),
             )
             ctx.tile_states.append((ckpt, stride))
             if whole:
@@ -130,10 +131,13 @@ class _HipScanFunction(torch.autograd.Function):
         if not whole:
             grads = [torch.empty(x.shape, dtype=k_in, device=x.device) if n else None for n in need]
         for (bs_, ds_), (ckpt, stride) in zip(ctx.tiles, ctx.tile_states):
-            h_tile = None if ctx.h_saved is None else ctx.h_saved[bs_, :, ds_]
+            if whole:
+                ops, h_tile = (xs, as_, bs, cs, dy), ctx.h_saved
+            else:
+                ops = tuple(t[bs_, :, ds_] for t in (xs, as_, bs, cs, dy))
+                h_tile = None if ctx.h_saved is None else ctx.h_saved[bs_, :, ds_]
             out = hip_scan.scan_backward(
-                xs[bs_, :, ds_], as_[bs_, :, ds_], bs[bs_, :, ds_], cs[bs_, :, ds_], dy[bs_, :, ds_],
-                h=h_tile, ckpt=None if h_tile is not None else ckpt, ckpt_stride=stride, need=need,
+                *ops, h=h_tile, ckpt=None if h_tile is not None else ckpt, ckpt_stride=stride, need=need,
             )
             if whole:
                 grads = list(out)
