@@ -249,6 +249,15 @@ int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int32_t ou
     }
     if (!fixed_t)
       while (threads > 256 && threads / 2 >= g && tiles(g, threads) < 2 * kCUs) threads >>= 1;
+    // Few chains and a long sequence (backward, 16-bit storage): every chain then has dozens of tiles in
+    // flight, its clusters are long and every tile reads the maps of the tiles before it.  Twice the
+    // chains at 256-byte row pieces is the better trade (B=1 L=65536 D=4096: 946 us against 998 us),
+    // even though the operands then all stay in registers.
+    if (direction == QSSM_BACKWARD && !fixed_g && es == 2 && g * vec * es == 512) {
+      const int64_t strips = (D + (int64_t)g * vec - 1) / ((int64_t)g * vec);
+      const int64_t seg = (int64_t)steps * (threads / g);
+      if ((int64_t)B * strips < 32 && L >= 256 * seg) g >>= 1;
+    }
     // Very short sequences: widen the rows instead of idling most time groups of a workgroup.
     if (!fixed_g)
       while (g < cap && g < threads && (int64_t)steps * (threads / g) / 2 >= lp2) g <<= 1;
