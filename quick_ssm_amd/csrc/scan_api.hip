@@ -249,11 +249,11 @@ int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int32_t ou
     }
     if (!fixed_t)
       while (threads > 256 && threads / 2 >= g && tiles(g, threads) < 2 * kCUs) threads >>= 1;
-    // Few chains and a long sequence (backward, 16-bit storage): every chain then has dozens of tiles in
-    // flight, its clusters are long and every tile reads the maps of the tiles before it.  Twice the
-    // chains at 256-byte row pieces is the better trade (B=1 L=65536 D=4096: 946 us against 998 us),
-    // even though the operands then all stay in registers.
-    if (direction == QSSM_BACKWARD && !fixed_g && es == 2 && g * vec * es == 512) {
+    // Few chains and a long sequence (16-bit storage): every chain then has dozens of tiles in flight, its
+    // clusters are long and every tile reads the maps of the tiles before it.  Twice the chains at 256-byte
+    // row pieces is the better trade (B=1 L=65536 D=4096: backward 932 us against 998 us, forward 531
+    // against 548).
+    if (!fixed_g && es == 2 && g * vec * es == 512) {
       const int64_t strips = (D + (int64_t)g * vec - 1) / ((int64_t)g * vec);
       const int64_t seg = (int64_t)steps * (threads / g);
       if ((int64_t)B * strips < 32 && L >= 256 * seg) g >>= 1;
@@ -400,7 +400,7 @@ int qssm_scan_forward_carry(const qssm_plan* plan, const void* x, qssm_strides s
   // c can live in LDS instead of registers when a row of the strip is one wavefront of 8-byte lanes
   // and c's rows can be fetched 16 bytes at a time.
   size_t lds = (size_t)plan->lds_bytes;
-  bool c_in_lds = y != nullptr && c != nullptr && es == 2 && v == 4 && plan->g_log2 == 6 && plan->steps == 8 &&
+  bool c_in_lds = y != nullptr && c != nullptr && es == 2 && v == 4 && (plan->g_log2 == 6 || plan->g_log2 == 5) && plan->steps == 8 &&
                   (plan->threads == 256 || plan->threads == 512) && ((uintptr_t)c) % 16 == 0 &&
                   (sc.b * es) % 16 == 0 && (sc.l * es) % 16 == 0 &&
                   lds + fwd_c_lds_bytes(plan->threads, plan->steps) <= (size_t)kMaxLdsBytes;
@@ -478,7 +478,7 @@ int qssm_scan_backward_carry(const qssm_plan* plan, const void* x, qssm_strides 
   // c and dy can live in LDS instead of registers when a row of the strip is one wavefront of 8-byte
   // lanes in both and their rows can be fetched 16 bytes at a time.
   size_t lds = (size_t)plan->lds_bytes;
-  bool cg_in_lds = es == 2 && os == 2 && v == 4 && plan->g_log2 == 6 && plan->steps == 8 && plan->threads == 256 &&
+  bool cg_in_lds = es == 2 && os == 2 && v == 4 && (plan->g_log2 == 6 || plan->g_log2 == 5) && plan->steps == 8 && plan->threads == 256 &&
                    ((uintptr_t)c) % 16 == 0 && (sc.b * es) % 16 == 0 && (sc.l * es) % 16 == 0 &&
                    ((uintptr_t)dy) % 16 == 0 && (sdy.b * os) % 16 == 0 && (sdy.l * os) % 16 == 0 &&
                    lds + bwd_cg_lds_bytes(plan->threads, plan->steps) <= (size_t)kMaxLdsBytes;

@@ -48,6 +48,10 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   int* sSeg = reinterpret_cast<int*>(sE + cols);
   char* sC = reinterpret_cast<char*>(sSeg) + 16 + ((int)threadIdx.x >> 6) * (T * 512);  // CLDS: this wave's [T rows][512 bytes] of c
   char* sG = sC + (NTH / 64) * (T * 512);                                  // and of dy
+  // Where step i of this lane sits in its wavefront's LDS block: the loads that fill it deposit 1024 bytes per
+  // instruction in lane order, i.e. per pair of steps [group in wavefront][step parity][G * 8 bytes].
+  const int lds_lane = (((int)threadIdx.x & 63) >> g.g_log2) * (G * 16) + ((int)threadIdx.x & (G - 1)) * 8;
+  auto lds_row = [&](int i) { return (i >> 1) * 1024 + (i & 1) * (G * 8); };
 
   const int tid = threadIdx.x;
   const int chain = blockIdx.x % g.n_chains;
@@ -117,10 +121,12 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
         rb[i] = load_stream<Tin, VEC>(bb, bo + i * bs);
         rx[i] = load_stream<Tin, VEC>(xb, xo + i * xs);
       }
-      // lanes 0-31 fetch one row of the strip (16 bytes each), lanes 32-63 the next one
+      // 16 bytes per lane: the first half of a lane group's lanes fetches one row of the strip, the second half
+      // the next one (64 lanes per row: a wavefront covers two rows of one group; 32: two rows of two groups)
       const int wl = tid & 63;
-      const char* csrc = cb + (uint32_t)(j * T + (wl >> 5)) * cs + (uint32_t)(wl & 31) * 16u;
-      const char* gsrc = gb + (uint32_t)(j * T + (wl >> 5)) * gs + (uint32_t)(wl & 31) * 16u;
+      const int half = (wl >> (g.g_log2 - 1)) & 1, piece = wl & ((G >> 1) - 1);
+      const char* csrc = cb + (uint32_t)(j * T + half) * cs + (uint32_t)piece * 16u;
+      const char* gsrc = gb + (uint32_t)(j * T + half) * gs + (uint32_t)piece * 16u;
 #pragma unroll
       for (int k = 0; k < T / 2; ++k) {
         __builtin_amdgcn_global_load_lds((global_ptr_t)(csrc + (uint32_t)(2 * k) * cs), (lds_ptr_t)(sC + k * 1024), 16, 0, 2);
@@ -174,8 +180,8 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
           cw = load_stream<Tin, VEC>(cb, co + i * cs);
           gw = load_stream<Tout, VEC>(gb, go + i * gs);
         }
-        *reinterpret_cast<Words<Tin, VEC>*>(sC + i * 512 + (tid & 63) * 8) = cw;
-        *reinterpret_cast<Words<Tout, VEC>*>(sG + i * 512 + (tid & 63) * 8) = gw;
+        *reinterpret_cast<Words<Tin, VEC>*>(sC + lds_row(i) + lds_lane) = cw;
+        *reinterpret_cast<Words<Tout, VEC>*>(sG + lds_row(i) + lds_lane) = gw;
       }
     }
   }
@@ -258,8 +264,8 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
     Words<Tin, VEC> cw;
     Words<Tout, VEC> gw;
     if (CLDS) {
-      cw = *reinterpret_cast<const Words<Tin, VEC>*>(sC + i * 512 + (tid & 63) * 8);
-      gw = *reinterpret_cast<const Words<Tout, VEC>*>(sG + i * 512 + (tid & 63) * 8);
+      cw = *reinterpret_cast<const Words<Tin, VEC>*>(sC + lds_row(i) + lds_lane);
+      gw = *reinterpret_cast<const Words<Tout, VEC>*>(sG + lds_row(i) + lds_lane);
     } else {
       cw = rc[i];
       gw = rg[i];
@@ -408,8 +414,8 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
     Words<Tin, VEC> cw;
     Words<Tout, VEC> gw;
     if (CLDS) {
-      cw = *reinterpret_cast<const Words<Tin, VEC>*>(sC + i * 512 + (tid & 63) * 8);
-      gw = *reinterpret_cast<const Words<Tout, VEC>*>(sG + i * 512 + (tid & 63) * 8);
+      cw = *reinterpret_cast<const Words<Tin, VEC>*>(sC + lds_row(i) + lds_lane);
+      gw = *reinterpret_cast<const Words<Tout, VEC>*>(sG + lds_row(i) + lds_lane);
     } else {
       cw = rc[i];
       gw = rg[i];

@@ -17,8 +17,8 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 // CLDS: the c operand is not needed before the last sweep, so it is loaded straight into LDS
 // (no destination registers) and read from there step by step: 16 VGPRs fewer across the
-// tile's whole life, which is one more resident workgroup per SIMD.  Needs 64 lanes per row and
-// 8 bytes per lane, so that one wavefront-wide 16-byte-per-lane load covers two rows of the strip.
+// tile's whole life, which is one more resident workgroup per SIMD.  Needs 64 or 32 lanes per row and
+// 8 bytes per lane, so that one wavefront-wide 16-byte-per-lane load covers whole rows of the strip.
 template <typename Tin, typename Tout, int VEC, int T, int NTH, bool CLDS>
 __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   static_assert(!CLDS || (sizeof(Tin) * VEC == 8 && T % 2 == 0), "LDS-resident c: 8 bytes per lane, even step count");
@@ -40,6 +40,10 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
 
   const int tid = threadIdx.x;
   const int chain = blockIdx.x % g.n_chains;
+  // Where step i of this lane sits in its wavefront's block of sC: the loads that fill it deposit 1024 bytes
+  // per instruction in lane order, i.e. per pair of steps [group in wavefront][step parity][G * 8 bytes].
+  const int lds_lane = ((tid & 63) >> g.g_log2) * (G * 16) + (tid & (G - 1)) * 8;
+  auto lds_row = [&](int i) { return (i >> 1) * 1024 + (i & 1) * (G * 8); };
 
   // ---- claim a tile of this chain, in time order -------------------------------------------
   int seg = 0;
@@ -103,9 +107,11 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
       rx[i] = load_stream<Tin, VEC>(xb, xo + i * xs);
     }
     if (CLDS) {
-      // lanes 0-31 fetch one row of the strip (16 bytes each), lanes 32-63 the next one
+      // 16 bytes per lane: the first half of a lane group's lanes fetches one row of the strip, the second half
+      // the next one (64 lanes per row: a wavefront covers two rows of one group; 32: two rows of two groups)
       const int wl = tid & 63;
-      const char* src = cb + (uint32_t)(j * T + (wl >> 5)) * cs + (uint32_t)(wl & 31) * 16u;
+      const int half = (wl >> (g.g_log2 - 1)) & 1, piece = wl & ((G >> 1) - 1);
+      const char* src = cb + (uint32_t)(j * T + half) * cs + (uint32_t)piece * 16u;
       char* dst = sC + (tid >> 6) * (T * 512);
 #pragma unroll
       for (int k = 0; k < T / 2; ++k)
@@ -135,12 +141,12 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
     if (CLDS) {
       // Ragged tile: c goes through a register one step at a time (rare, and kept rolled up so that
       // it does not bring the sixteen registers back).
-      char* dst = sC + (tid >> 6) * (T * 512) + (tid & 63) * 8;
+      char* dst = sC + (tid >> 6) * (T * 512) + lds_lane;
 #pragma unroll 1
       for (int i = 0; i < T; ++i) {
         Words<Tin, VEC> cw = fill_words<Tin, VEC>(false);
         if (dok && t0 + i < g.L) cw = load_stream<Tin, VEC>(cb, co + i * cs);
-        *reinterpret_cast<Words<Tin, VEC>*>(dst + i * 512) = cw;
+        *reinterpret_cast<Words<Tin, VEC>*>(dst + lds_row(i)) = cw;
       }
     }
   }
@@ -315,7 +321,7 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   for (int i = 0; i < T; ++i) {
     float yv[VEC];
     Words<Tin, VEC> cw;
-    if (CLDS) cw = *reinterpret_cast<const Words<Tin, VEC>*>(sC + (tid >> 6) * (T * 512) + i * 512 + (tid & 63) * 8);
+    if (CLDS) cw = *reinterpret_cast<const Words<Tin, VEC>*>(sC + (tid >> 6) * (T * 512) + lds_row(i) + lds_lane);
     else cw = rc[i];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {

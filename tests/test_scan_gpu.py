@@ -134,15 +134,16 @@ def test_fp32_output_from_16bit_operands(gpu, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+@pytest.mark.parametrize("g_log2", [6, 5], ids=["rows64", "rows32"])
 @pytest.mark.parametrize("shape", [(2, 700, 512), (2, 1100, 264), (1, 97, 256)], ids=lambda s: "x".join(map(str, s)))
-def test_lds_resident_operands_and_register_path_agree(gpu, dtype, shape):
-    # 64-lane rows whose bytes are 16-byte aligned take the kernels that load c (and dy) straight into LDS; the
-    # same values at an offset of 4 elements take the register-only kernels.  Both must meet the oracle: ragged last
-    # tiles, a partial second strip, checkpoint on and off, y in the operands' storage and in fp32.
+def test_lds_resident_operands_and_register_path_agree(gpu, dtype, shape, g_log2):
+    # 64- or 32-lane rows whose bytes are 16-byte aligned take the kernels that load c (and dy) straight into LDS;
+    # the same values at an offset of 4 elements take the register-only kernels.  Both must meet the oracle: ragged
+    # last tiles, a partial last strip, checkpoint on and off, y in the operands' storage and in fp32.
     B, L, D = shape
     x, a, b, c, dy = make_inputs(shape, dtype=dtype, seed=31)
     ref = oracle_all(x, a, b, c, dy)
-    tune = 7 | (8 << 8)  # 64 lanes per row, 8 steps per lane; workgroup size and clusters automatic
+    tune = (g_log2 + 1) | (8 << 8)  # lanes per row, 8 steps per lane; workgroup size and clusters automatic
 
     def run(place, out_dtype=dtype, gy=dy, keep_h=False):
         ops = [place(t) for t in (x, a, b, c)]
@@ -165,8 +166,8 @@ def test_lds_resident_operands_and_register_path_agree(gpu, dtype, shape):
     assert all(t.data_ptr() % 16 == 0 for t in ops)
     fwd_plan = hip_scan.make_plan(B, L, D, dtype, dtype, _lib.QSSM_FORWARD, 8, 32, tune)
     bwd_plan = hip_scan.make_plan(B, L, D, dtype, dtype, _lib.QSSM_BACKWARD, 8, 0, tune)
-    assert (fwd_plan.g_log2, fwd_plan.vec, fwd_plan.steps) == (6, 4, 8) and fwd_plan.threads in (256, 512)
-    assert (bwd_plan.g_log2, bwd_plan.vec, bwd_plan.steps, bwd_plan.threads) == (6, 4, 8, 256)
+    assert (fwd_plan.g_log2, fwd_plan.vec, fwd_plan.steps) == (g_log2, 4, 8) and fwd_plan.threads in (256, 512)
+    assert (bwd_plan.g_log2, bwd_plan.vec, bwd_plan.steps, bwd_plan.threads) == (g_log2, 4, 8, 256)
     _check_all(got_lds, ref, TOL[dtype])
     _check_all(run(aligned, keep_h=True)[0], ref, TOL[dtype])
 
