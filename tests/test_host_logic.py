@@ -233,3 +233,28 @@ def test_plan_invariants_over_random_shapes(hip_lib):
             assert (p.workspace_bytes >= words if p.n_seg > 1 else p.workspace_bytes == 0), what
             assert p.ckpt_elems == B * p.n_ckpt * D and p.n_ckpt == -(-L // p.ckpt_stride), what
         assert fwd.ckpt_stride == bwd.ckpt_stride == bwd.seg_len
+
+
+def test_tile_index_arithmetic_over_random_shapes(hip_lib):
+    # the same bounds model over a seeded sweep of small shapes, alignments, storage types and forced geometries
+    import random
+    rng = random.Random(99)
+    for _ in range(60):
+        B = rng.choice([1, 2, 3])
+        L = rng.choice([1, 5, 31, 32, 33, 64, 65, 127, 200, 513, 1030])
+        D = rng.choice([1, 2, 4, 6, 8, 20, 64, 72, 128, 136, 260, 512])
+        dtype = rng.choice([torch.float32, torch.float16, torch.bfloat16])
+        align = rng.choice([1, 2, 4, 8])
+        g = rng.choice([0, 0, 4, 5, 6, 7, 8])                      # automatic, or 8 .. 128 lanes per row
+        tune = g | (rng.choice([0, 4, 8]) << 8) | (rng.choice([0, 1, 2]) << 24) | (rng.choice([0, 1, 2, 3, 4]) << 28)
+        for direction in (_lib.QSSM_BACKWARD, _lib.QSSM_FORWARD):
+            try:
+                plan = hip_scan.make_plan(B, L, D, dtype, dtype, direction, align, 0, tune)
+            except Exception as exc:   # a forced geometry the planner refuses is fine; anything else is not
+                assert "LDS" in str(exc) or "ckpt_stride" in str(exc), (B, L, D, dtype, align, tune, str(exc))
+                continue
+            lo, hi, hi_ckpt, hi_word = _tile_accesses(plan, B, L, D)
+            what = (B, L, D, dtype, align, tune, plan.describe())
+            assert lo >= 0 and hi == B * L * D - 1, what
+            assert hi_ckpt < plan.ckpt_elems, what
+            assert hi_word <= plan.workspace_bytes, what

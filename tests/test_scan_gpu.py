@@ -612,3 +612,42 @@ def test_calibration_copy_moves_every_byte(gpu):
         assert lib.qssm_copy_bytes(dst.data_ptr(), src.data_ptr(), nbytes, stream) == 0
         assert torch.equal(dst[:nbytes], src) and int(dst[nbytes:].sum()) == 0
     assert lib.qssm_copy_bytes(None, None, 0, stream) == 0
+
+
+def test_random_shapes_layouts_and_storage_against_oracle(gpu):
+    # a seeded sweep: shapes around the tile and strip boundaries, every built storage pair, operands that are
+    # contiguous, column slices of a wider tensor, or every second time step of a longer one; checkpoint on and off
+    import random
+    rng = random.Random(7)
+    pairs = [(torch.float32, torch.float32), (torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16),
+             (torch.float16, torch.float32), (torch.bfloat16, torch.float32)]
+    for case in range(36):
+        B = rng.choice([1, 2, 3])
+        L = rng.choice([1, 2, 31, 33, 64, 65, 129, 255, 300, 513, 1030])
+        D = rng.choice([1, 3, 4, 8, 12, 64, 100, 128, 256, 264, 520])
+        dtype, out_dtype = rng.choice(pairs)
+        layout = rng.choice(["dense", "columns", "steps"])
+        checkpoint = rng.random() < 0.7
+        print(f"case {case}: B{B} L{L} D{D} {dtype} -> {out_dtype} {layout} checkpoint={checkpoint}", flush=True)
+        x, a, b, c, dy = make_inputs((B, L, D), dtype=dtype, seed=1000 + case, out_dtype=out_dtype)
+        ref = oracle_all(x, a, b, c, dy)
+
+        def place(t):
+            if layout == "columns":      # a column slice: row stride D + 16, first column at 8
+                wide = torch.zeros(B, L, D + 16, dtype=t.dtype, device=gpu)
+                wide[:, :, 8:8 + D] = t.to(gpu)
+                return wide[:, :, 8:8 + D]
+            if layout == "steps":        # every second step of a sequence twice as long
+                long = torch.zeros(B, 2 * L, D, dtype=t.dtype, device=gpu)
+                long[:, ::2] = t.to(gpu)
+                return long[:, ::2]
+            return t.to(gpu)
+
+        leaves = [place(t).detach().requires_grad_(True) for t in (x, a, b, c)]
+        y = scan(*leaves, checkpoint=checkpoint, out_dtype=out_dtype)
+        y.backward(place(dy))
+        assert hip_scan.workspace_status() == 0
+        tol_y, tol_g = TOL[out_dtype], TOL[dtype]
+        assert_close(f"case {case} y", y.detach().cpu(), ref["y"], tol_y)
+        for name, leaf in zip(("dx", "da", "db", "dc"), leaves):
+            assert_close(f"case {case} {name}", leaf.grad.cpu(), ref[name], tol_g)
