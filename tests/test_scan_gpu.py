@@ -651,3 +651,26 @@ def test_random_shapes_layouts_and_storage_against_oracle(gpu):
         assert_close(f"case {case} y", y.detach().cpu(), ref["y"], tol_y)
         for name, leaf in zip(("dx", "da", "db", "dc"), leaves):
             assert_close(f"case {case} {name}", leaf.grad.cpu(), ref[name], tol_g)
+
+
+def test_nan_in_an_input_stays_in_its_column_and_nothing_hangs(gpu):
+    # one NaN in x: from that step on y, da and dc of that column are NaN (the state carries it), db only at that
+    # step, dx nowhere; every other column is untouched, no tile waits for ever (the tags of the exchanged words
+    # do not depend on their payload), and the pattern is the oracle's
+    shape = (2, 600, 260)
+    x, a, b, c, dy = make_inputs(shape, dtype=torch.bfloat16, seed=77)
+    x[0, 100, 5] = float("nan")
+    got = run_scan_with_grads(scan, x, a, b, c, dy, gpu, checkpoint=True)
+    assert hip_scan.workspace_status() == 0
+    ref = oracle_all(x, a, b, c, dy)
+    for name in ("y", "dx", "da", "db", "dc"):
+        g = got[name].float().numpy()
+        r = np.asarray(ref[name], dtype=np.float64)
+        assert np.array_equal(np.isnan(g), np.isnan(r)), name
+        ok = ~np.isnan(r)
+        scale = np.abs(r[ok]).max()
+        assert np.abs(g[ok] - r[ok]).max() <= TOL[torch.bfloat16] * scale, name
+    y = got["y"].float()
+    assert torch.isnan(y[0, 100:, 5]).all() and torch.isfinite(y[0, :100, 5]).all()
+    assert torch.isfinite(got["dx"].float()).all()
+    assert int(torch.isnan(got["db"].float()).sum()) == 1
