@@ -538,13 +538,14 @@ def _rows_check(got, ops, dy, rows, tol):
 
 
 def test_config1_bf16_full_shape(gpu):
-    # B=8 L=4096 D=2048 bf16: batch rows 0 and 7 against the oracle over every tile of their chains, the
-    # rest through properties that hold at any size
+    # B=8 L=4096 D=2048 bf16: every batch row of every output against the oracle, plus the properties that hold at
+    # any size
     shape = (8, 4096, 2048)
     x, a, b, c, dy = make_inputs(shape, dtype=torch.bfloat16, seed=0)
     print("case config1 full shape", flush=True)
     got = run_scan_with_grads(scan, x, a, b, c, dy, gpu, block_l=256, checkpoint=True)
-    _rows_check(got, (x, a, b, c), dy, (0, 7), TOL[torch.bfloat16])
+    assert hip_scan.workspace_status() == 0
+    _rows_check(got, (x, a, b, c), dy, range(shape[0]), TOL[torch.bfloat16])
     assert torch.all(got["da"][:, 0, :] == 0)
     for k in got:
         assert torch.isfinite(got[k].float()).all(), k
@@ -559,24 +560,150 @@ def test_config1_bf16_full_shape(gpu):
     assert hip_scan.workspace_status() == 0
 
 
+@pytest.mark.timeout(600)
 def test_config2_fp16_long_sequence_near_unit_decay(gpu):
-    # B=1 L=65536 D=4096 fp16, a in [0.99, 1], block_l=1024, tile_d=1024: first and last 64 columns over all of L
+    # B=1 L=65536 D=4096 fp16, a in [0.99, 1], block_l=1024, tile_d=1024: every column over all of L, the oracle
+    # taking 512 columns at a time
     shape = (1, 65536, 4096)
     x, a, b, c, dy = make_inputs(shape, dtype=torch.float16, seed=1, a_lo=0.99, a_span=0.01)
     print("case config2 full shape", flush=True)
     got = run_scan_with_grads(scan, x, a, b, c, dy, gpu, block_l=1024, checkpoint=True, tile_d=1024)
-    for cols in (slice(0, 64), slice(4032, 4096)):
+    assert hip_scan.workspace_status() == 0
+    for k in got:
+        assert torch.isfinite(got[k].float()).all(), k
+    for c0 in range(0, shape[2], 512):
+        cols = slice(c0, c0 + 512)
+        print(f"  columns {c0}:{c0 + 512}", flush=True)
         ref = oracle_all(x[..., cols], a[..., cols], b[..., cols], c[..., cols], dy[..., cols])
         for k in ("y", "dx", "da", "db", "dc"):
             assert_close(f"{k}[cols {cols.start}:{cols.stop}]", got[k][..., cols], ref[k], TOL[torch.float16])
-    for k in got:
-        assert torch.isfinite(got[k].float()).all(), k
+
+
+@pytest.mark.timeout(600)
+def test_config3_scan_at_its_own_shape(gpu):
+    # the scan inside the config-3 layer: B=16 L=2048 D=4096, fp16 operands, fp32 y and dy, checkpoint=True.
+    # Every batch row against the oracle: 1e-5 for y (fp32 storage), 1e-2 for the gradients (fp16 storage).
+    shape = (16, 2048, 4096)
+    x, a, b, c, dy = make_inputs(shape, dtype=torch.float16, seed=3, out_dtype=torch.float32)
+    print("case config3 scan full shape", flush=True)
+    got = run_scan_with_grads(scan, x, a, b, c, dy, gpu, block_l=256, checkpoint=True, out_dtype=torch.float32)
     assert hip_scan.workspace_status() == 0
+    assert got["y"].dtype == torch.float32 and got["dx"].dtype == torch.float16
+    for r in range(shape[0]):
+        sl = slice(r, r + 1)
+        ref = oracle_all(x[sl], a[sl], b[sl], c[sl], dy[sl])
+        assert_close(f"y[row {r}]", got["y"][sl], ref["y"], TOL[torch.float32])
+        for k in ("dx", "da", "db", "dc"):
+            assert_close(f"{k}[row {r}]", got[k][sl], ref[k], TOL[torch.float16])
+    assert torch.all(got["da"][:, 0, :] == 0)
 
 
-def test_config3_ssm_layer_matches_sequential_path(gpu):
-    # SSM(hidden, state = 4*hidden), fp32 parameters, fp16 scan operands, fp32 scan output; the device layer
-    # against the same layer on the sequential torch path (smaller than config 3 so the CPU side takes seconds)
+def _layer_oracle_f64(layer, xin, gout, gemm_device):
+    """float64 composition of the committed oracles for one SSM layer step (quick_ssm/layers.py:60-107):
+    rmsnorm_oracle -> float64 projections -> gates_oracle -> scan oracle -> float64 out projection (+ residual),
+    and the same chain backwards.  The operands of the scan are rounded to `compute_dtype` where the layer rounds
+    them (layers.py:85-88), so the scan oracle sees the stored values the kernels see up to the rounding of
+    values within an ulp of a tie.  The matrix products (torch's library GEMM on both sides of the comparison, not
+    part of the path under test) run in float64 on `gemm_device`; everything elementwise runs on the CPU oracles.
+    """
+    from oracle import gates_oracle, rmsnorm_oracle
+
+    f64 = torch.float64
+    P = {n: p.detach().to("cpu", f64) for n, p in layer.named_parameters()}
+    B, L, H = xin.shape
+    S = layer.state_size_dim
+    x64 = xin.detach().to("cpu", f64)
+    eps = layer.pre_norm.eps
+    u = torch.from_numpy(rmsnorm_oracle.rmsnorm_forward_f64(x64.numpy(), P["pre_norm.weight"].numpy(), eps))
+
+    def mm(lhs, rhs):
+        return (lhs.to(gemm_device) @ rhs.to(gemm_device)).cpu()
+
+    u2 = u.reshape(-1, H)
+    pre = {n: mm(u2, P[f"{n}.weight"].t()) for n in ("A_proj", "B_proj", "C_proj_a", "C_proj_b", "D_proj")}
+    pre["A_proj"] = pre["A_proj"] + P["A_proj.bias"]
+    ga, gx, gc, gb = gates_oracle.gates_forward_f64(pre["A_proj"].numpy(), pre["B_proj"].numpy(),
+                                                    pre["C_proj_a"].numpy(), pre["C_proj_b"].numpy(),
+                                                    pre["D_proj"].numpy())
+    cd = layer.compute_dtype
+    ops = [torch.from_numpy(t).to(cd).reshape(B, L, S) for t in (gx, ga, gb, gc)]   # x, a, b, c as stored
+    _, y = oracle.forward_f64(*ops)
+    y2 = torch.from_numpy(y).reshape(-1, S)
+    out = (mm(y2, P["out_proj.weight"].t()) + P["out_proj.bias"]).reshape(B, L, H) + x64
+
+    g2 = gout.detach().to("cpu", f64).reshape(-1, H)
+    grads = {"out_proj.bias": g2.sum(0), "out_proj.weight": mm(g2.t(), y2)}
+    dy = mm(g2, P["out_proj.weight"])                                             # [rows, S]
+    dx_s, da_s, db_s, dc_s = oracle.backward_f64(*ops, dy.reshape(B, L, S).float())
+    # the scan's dy is the fp32 tensor autograd hands it; the oracle takes stored values
+    dpre = gates_oracle.gates_backward_f64(da_s.reshape(-1, S), dx_s.reshape(-1, S), dc_s.reshape(-1, S),
+                                           db_s.reshape(-1, S), pre["A_proj"].numpy(), pre["C_proj_a"].numpy(),
+                                           pre["C_proj_b"].numpy(), pre["D_proj"].numpy())
+    du = torch.zeros_like(u2)
+    for n, g in zip(("A_proj", "B_proj", "C_proj_a", "C_proj_b", "D_proj"), dpre):
+        g = torch.from_numpy(np.ascontiguousarray(g))
+        grads[f"{n}.weight"] = mm(g.t(), u2)
+        if n == "A_proj":
+            grads["A_proj.bias"] = g.sum(0)
+        du += mm(g, P[f"{n}.weight"])
+    dxn, dw = rmsnorm_oracle.rmsnorm_backward_f64(du.reshape(B, L, H).numpy(), x64.numpy(),
+                                                  P["pre_norm.weight"].numpy(), eps)
+    grads["pre_norm.weight"] = torch.from_numpy(dw)
+    dx = torch.from_numpy(dxn) + gout.detach().to("cpu", f64)
+    return out, dx, grads
+
+
+def _run_layer(mod, inp, gout):
+    mod.zero_grad(set_to_none=True)
+    inp = inp.clone().requires_grad_(True)
+    out = mod(inp)
+    out.backward(gout.to(inp.device))
+    grads = {n: p.grad.detach().cpu().clone() for n, p in mod.named_parameters()}
+    return out.detach().cpu(), inp.grad.detach().cpu(), grads
+
+
+def test_ssm_layer_small_matches_oracle_composition(gpu):
+    # the layer's whole step at a size the CPU does in a second, against the float64 composition of the oracles
+    from quick_ssm_amd.layers import SSM
+
+    torch.manual_seed(0)
+    layer = SSM(hidden_size=64, state_size_mult=4.0, compute_dtype=torch.float16, dtype=torch.float32).to(gpu)
+    xin = torch.randn(2, 192, 64)
+    gout = torch.randn(2, 192, 64)
+    out, dx, grads = _run_layer(layer, xin.to(gpu), gout)
+    assert hip_scan.workspace_status() == 0
+    ref_out, ref_dx, ref_grads = _layer_oracle_f64(layer, xin, gout, "cpu")
+    assert_close("layer out", out, ref_out.numpy(), 1e-2)
+    assert_close("layer dx", dx, ref_dx.numpy(), 1e-2)
+    for n in ref_grads:
+        assert_close(f"grad {n}", grads[n], ref_grads[n].numpy(), 1e-2)
+
+
+@pytest.mark.timeout(900)
+def test_config3_ssm_layer_at_its_own_shape(gpu):
+    # SSM(hidden 1024, state 4096), fp32 parameters, fp16 scan operands, fp32 scan output, B=16 L=2048, seeded
+    # default initialisation (quick_ssm/layers.py:31-58) and N(0,1) activations: output, input gradient and every
+    # parameter gradient against the float64 composition of the oracles (float64 GEMMs on the GPU: 5 TFLOP).
+    from quick_ssm_amd.layers import SSM
+
+    torch.manual_seed(0)
+    layer = SSM(hidden_size=1024, state_size_mult=4.0, compute_dtype=torch.float16, dtype=torch.float32).to(gpu)
+    g = torch.Generator(device="cpu").manual_seed(5)
+    xin = torch.randn(16, 2048, 1024, generator=g)
+    gout = torch.randn(16, 2048, 1024, generator=g)
+    print("case config3 layer full shape", flush=True)
+    out, dx, grads = _run_layer(layer, xin.to(gpu), gout)
+    assert hip_scan.workspace_status() == 0
+    ref_out, ref_dx, ref_grads = _layer_oracle_f64(layer, xin, gout, gpu)
+    assert_close("layer out", out, ref_out.numpy(), 1e-2)
+    assert_close("layer dx", dx, ref_dx.numpy(), 1e-2)
+    for n in ref_grads:
+        assert_close(f"grad {n}", grads[n], ref_grads[n].numpy(), 1e-2)
+
+
+def test_ssm_layer_matches_sequential_path(gpu):
+    # the device layer against the same layer on the product's sequential torch path (pinned on the reference's CPU
+    # path by tests/test_oracle.py)
     from quick_ssm_amd.layers import SSM
 
     torch.manual_seed(0)
