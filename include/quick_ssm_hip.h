@@ -173,6 +173,33 @@ QSSM_API int qssm_scan_forward(const qssm_plan* plan,
                       void* stream);
 
 /*
+ * Forward scan for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): qssm_scan_forward without the control block, workspace and epoch
+ * arguments.  Both buffers live in one array of QSSM_STATIC_SCRATCH_BYTES inside the library's device image;
+ * every GPU the library runs on holds its own copy until the process ends.  The call allocates nothing and
+ * never synchronises; its first call on a device looks the array's address up (make that call outside a
+ * capture).  Launches number themselves in the array (as with epoch 0), so a captured call replays correctly.
+ *   - Shapes whose plan needs more than 256 KiB of control block (4095 chains) or more workspace than the rest
+ *     of the array are refused with QSSM_EWORKSPACE; the headline shape (bf16, B=8 L=4096 D=2048: 20 MiB) fits.
+ *   - All calls on one GPU share that GPU's array: they must be ordered on one stream (or otherwise not
+ *     overlap); calls that overlap on one GPU race.  The array keeps the last call's words, which their flag
+ *     values make harmless; status word and ticket counters are cleared at the start of every call.
+ * Results are those of qssm_scan_forward for the same plan, bit for bit.
+ * No counterpart in the reference (its Triton launches allocate their scratch through torch,
+ * quick_ssm/triton_forwards.py:150-156); it exists for the callers named above.
+ */
+#define QSSM_STATIC_SCRATCH_BYTES (32u << 20)
+QSSM_API int qssm_scan_forward_static(const qssm_plan* plan,
+                             const void* x, qssm_strides sx,
+                             const void* a, qssm_strides sa,
+                             const void* b, qssm_strides sb,
+                             const void* c, qssm_strides sc,
+                             void* y, qssm_strides sy,
+                             float* h_out, qssm_strides sh,
+                             float* ckpt,
+                             void* stream);
+
+/*
  * Forward scan with a carried state: the same launch, started from `h_init` instead of zero and/or
  * reporting the state after the last step, so that a sequence can be scanned in pieces (chunked
  * prefill, token-by-token generation) with results identical to one scan over the whole of it.

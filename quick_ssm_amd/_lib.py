@@ -17,6 +17,7 @@ LIB_PATH = Path(__file__).resolve().parent / LIB_NAME
 QSSM_F32, QSSM_F16, QSSM_BF16 = 0, 1, 2
 QSSM_FORWARD, QSSM_BACKWARD = 0, 1
 QSSM_RMSNORM_MIN_PARTIAL_ROWS = 8
+QSSM_STATIC_SCRATCH_BYTES = 32 << 20
 QSSM_EINVAL, QSSM_EALIGN, QSSM_EWORKSPACE, QSSM_ESTATE = -1, -2, -3, -4
 
 EXPORTED_SYMBOLS = (
@@ -29,6 +30,7 @@ EXPORTED_SYMBOLS = (
     "qssm_scan_backward",
     "qssm_scan_forward_carry",
     "qssm_scan_backward_carry",
+    "qssm_scan_forward_static",
     "qssm_gates_forward",
     "qssm_gates_backward",
     "qssm_rmsnorm_forward",
@@ -102,6 +104,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.qssm_scan_forward.argtypes = (
         [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, u64, vp, u64, ctypes.c_uint32, vp]
     )
+    lib.qssm_scan_forward_static.restype = ctypes.c_int
+    lib.qssm_scan_forward_static.argtypes = [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp]
     lib.qssm_scan_backward.restype = ctypes.c_int
     lib.qssm_scan_backward.argtypes = (
         [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, Strides] * 4 + [vp, u64, vp, u64, ctypes.c_uint32, vp]

@@ -5,6 +5,7 @@
 #include <string.h>
 
 #include <initializer_list>
+#include <mutex>
 #include <utility>
 
 #include "scan_common.h"
@@ -135,10 +136,13 @@ static bool tile_span_ok(const qssm_plan* pl, const void* p, int64_t sb, int64_t
 // One lane behind every launch that uses device-counted epochs: the next launch on the stream gets
 // the next flag value.  A kernel of its own, so that every workgroup of the scan has read the
 // count before it changes, and so that a captured graph replays correctly (the count lives in device
-// memory, not in a kernel argument).  The count never takes the value whose successor is zero.
-__global__ void count_launch_kernel(unsigned* count) {
-  const unsigned next = *count + 1u;
-  *count = next == 0xffffffffu ? 0u : next;
+// memory, not in a kernel argument).  The count never takes the value whose successor is zero: from
+// `reset_at` on it starts again at zero (the caller-owned buffers wrap at the end of the 32-bit range;
+// the library's own scratch array wraps earlier, after its workspace has been wiped).
+static const unsigned kCountWrapAt = 0xfffffffeu;
+__global__ void count_launch_kernel(unsigned* count, unsigned reset_at) {
+  const unsigned cur = *count;
+  *count = cur >= reset_at ? 0u : cur + 1u;
 }
 
 static void fill_geometry(Geometry* g, const qssm_plan* pl, void* control, void* workspace, uint32_t epoch) {
@@ -168,6 +172,12 @@ static void fill_geometry(Geometry* g, const qssm_plan* pl, void* control, void*
 }  // namespace qssm
 
 using namespace qssm;
+
+static int forward_launch(const qssm_plan* plan, const void* x, qssm_strides sx, const void* a, qssm_strides sa,
+                          const void* b, qssm_strides sb, const void* c, qssm_strides sc, void* y, qssm_strides sy,
+                          float* h_out, qssm_strides sh, float* ckpt, const float* h_init, float* h_final,
+                          void* control, uint64_t control_size, void* workspace, uint64_t workspace_bytes,
+                          uint32_t epoch, unsigned count_reset_at, void* stream);
 
 extern "C" {
 
@@ -361,6 +371,17 @@ int qssm_scan_forward_carry(const qssm_plan* plan, const void* x, qssm_strides s
                             float* h_out, qssm_strides sh, float* ckpt, const float* h_init, float* h_final,
                             void* control, uint64_t control_size, void* workspace, uint64_t workspace_bytes,
                             uint32_t epoch, void* stream) {
+  return forward_launch(plan, x, sx, a, sa, b, sb, c, sc, y, sy, h_out, sh, ckpt, h_init, h_final, control,
+                        control_size, workspace, workspace_bytes, epoch, kCountWrapAt, stream);
+}
+
+}  // extern "C"
+
+static int forward_launch(const qssm_plan* plan, const void* x, qssm_strides sx, const void* a, qssm_strides sa,
+                          const void* b, qssm_strides sb, const void* c, qssm_strides sc, void* y, qssm_strides sy,
+                          float* h_out, qssm_strides sh, float* ckpt, const float* h_init, float* h_final,
+                          void* control, uint64_t control_size, void* workspace, uint64_t workspace_bytes,
+                          uint32_t epoch, unsigned count_reset_at, void* stream) {
   int rc = check_plan(plan, QSSM_FORWARD);
   if (rc != 0) return rc;
   if (plan->B == 0 || plan->L == 0 || plan->D == 0) return 0;
@@ -409,10 +430,12 @@ int qssm_scan_forward_carry(const qssm_plan* plan, const void* x, qssm_strides s
     return fail(QSSM_EINVAL, "no forward kernel for vec=%d steps=%d threads=%d", plan->vec, plan->steps, plan->threads);
   if (epoch == 0 && plan->n_seg > 1)
     hipLaunchKernelGGL(count_launch_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream,
-                       (unsigned*)((char*)control + kLaunchCountOffset));
+                       (unsigned*)((char*)control + kLaunchCountOffset), count_reset_at);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : hip_fail(e, "scan_fwd_kernel launch");
 }
+
+extern "C" {
 
 int qssm_scan_backward(const qssm_plan* plan, const void* x, qssm_strides sx, const void* a, qssm_strides sa,
                        const void* b, qssm_strides sb, const void* c, qssm_strides sc, const void* dy,
@@ -487,7 +510,7 @@ int qssm_scan_backward_carry(const qssm_plan* plan, const void* x, qssm_strides 
     return fail(QSSM_EINVAL, "no backward kernel for vec=%d steps=%d threads=%d", plan->vec, plan->steps, plan->threads);
   if (epoch == 0 && plan->n_seg > 1)
     hipLaunchKernelGGL(count_launch_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream,
-                       (unsigned*)((char*)control + kLaunchCountOffset));
+                       (unsigned*)((char*)control + kLaunchCountOffset), kCountWrapAt);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : hip_fail(e, "scan_bwd_kernel launch");
 }
@@ -580,6 +603,83 @@ int qssm_rmsnorm_backward(const void* dy, int64_t ld_dy, const void* x, int64_t 
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : hip_fail(e, "rmsnorm_bwd_kernel launch");
 }
+
+}  // extern "C"
+
+// ---- the forward scan for callers that cannot allocate ----------------------------------------------------
+//
+// Control block and workspace of this entry point live in one array in the library's device image: nothing is
+// allocated, by the caller or here.  Every GPU the library runs on holds its own copy of the array, at its own
+// address, until the process ends.  `g_scratch` below is only the host-side handle of that array: its device
+// address is asked for once per device (hipGetSymbolAddress) and kept in g_scratch_ptr; host code uses that
+// pointer wherever it needs the array's memory.
+static const uint64_t kScratchControlBytes = 256u << 10;                  // status, count, up to 4095 chains
+static const uint64_t kScratchBytes = (uint64_t)QSSM_STATIC_SCRATCH_BYTES;  // control block + workspace
+static const unsigned kScratchWipeAt = 0xfffffff0u;  // launch count from which the array is wiped and the count restarts
+static __device__ __align__(256) unsigned char g_scratch[QSSM_STATIC_SCRATCH_BYTES];
+
+static const int kMaxDevices = 64;
+static unsigned char* g_scratch_ptr[kMaxDevices];   // per device: where that device keeps the array
+static std::mutex g_scratch_mutex;
+
+// Before every launch on the array: status word and ticket counters back to zero (a launch that failed may have
+// left them dirty), the launch count kept.  Once the count has reached kScratchWipeAt the words of the whole
+// array are cleared as well, and the counting kernel behind the scan then restarts the count, so that no word of
+// an old launch can ever carry the flag value of a new one.  Every workgroup reads the count before anyone
+// rewrites the word beside it with the same value.
+__global__ void __launch_bounds__(256) scratch_prologue_kernel(uint4* scratch, uint64_t control16, uint64_t total16) {
+  const unsigned count = reinterpret_cast<const unsigned*>(scratch)[kLaunchCountOffset / 4];
+  const uint64_t n16 = count >= kScratchWipeAt ? total16 : control16;
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride)
+    scratch[i] = i == 0 ? make_uint4(0u, count, 0u, 0u) : make_uint4(0u, 0u, 0u, 0u);
+}
+
+static int scratch_for_current_device(unsigned char** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+  if (dev < 0 || dev >= kMaxDevices) return fail(QSSM_EINVAL, "device index %d beyond the %d this entry point keeps", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_scratch));
+    if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+    if (p == nullptr || ((uintptr_t)p) % 256 != 0) return fail(QSSM_EINVAL, "scratch array has no usable device address");
+    g_scratch_ptr[dev] = static_cast<unsigned char*>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
+extern "C" int qssm_scan_forward_static(const qssm_plan* plan, const void* x, qssm_strides sx, const void* a,
+                                        qssm_strides sa, const void* b, qssm_strides sb, const void* c,
+                                        qssm_strides sc, void* y, qssm_strides sy, float* h_out, qssm_strides sh,
+                                        float* ckpt, void* stream) {
+  int rc = check_plan(plan, QSSM_FORWARD);
+  if (rc != 0) return rc;
+  if (plan->B == 0 || plan->L == 0 || plan->D == 0) return 0;
+  if (plan->control_bytes > kScratchControlBytes || plan->workspace_bytes > kScratchBytes - kScratchControlBytes)
+    return fail(QSSM_EWORKSPACE,
+                "shape needs %llu bytes of control block and %llu of workspace; the built-in scratch array holds %llu "
+                "and %llu: use qssm_scan_forward with buffers of the caller",
+                (unsigned long long)plan->control_bytes, (unsigned long long)plan->workspace_bytes,
+                (unsigned long long)kScratchControlBytes, (unsigned long long)(kScratchBytes - kScratchControlBytes));
+  unsigned char* scratch = nullptr;
+  rc = scratch_for_current_device(&scratch);
+  if (rc != 0) return rc;
+  if (plan->n_seg > 1) {
+    hipLaunchKernelGGL(scratch_prologue_kernel, dim3(64), dim3(256), 0, (hipStream_t)stream,
+                       reinterpret_cast<uint4*>(scratch), (uint64_t)(plan->control_bytes + 15) / 16, kScratchBytes / 16);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e, "scratch_prologue_kernel launch");
+  }
+  return forward_launch(plan, x, sx, a, sa, b, sb, c, sc, y, sy, h_out, sh, ckpt, nullptr, nullptr, scratch,
+                        kScratchControlBytes, scratch + kScratchControlBytes, kScratchBytes - kScratchControlBytes,
+                        /*epoch=*/0, kScratchWipeAt, stream);
+}
+
+extern "C" {
 
 int qssm_copy_bytes(void* dst, const void* src, uint64_t bytes, void* stream) {
   if (bytes == 0) return 0;
