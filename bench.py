@@ -104,8 +104,6 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--tune-fwd", type=int, default=0, help="geometry override for sweeps (see qssm_plan_scan)")
-    ap.add_argument("--tune-bwd", type=int, default=0)
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -156,26 +154,28 @@ def main() -> int:
         for t in ops:
             t.grad = None
         y = scan(*ops, block_l=block_l, checkpoint=True, out_dtype=out_dtype)
-        y.backward(gy)
+        # one device, one graph: run the backward on this thread instead of waking autograd's device thread (the
+        # hand-over costs more than the launch it brackets when the workload is small; it changes nothing on the GPU)
+        with torch.autograd.set_multithreading_enabled(False):
+            y.backward(gy)
 
     # ---- the two kernels on their own, through the C ABI -------------------------------------------
     # Measured first: the device's power management takes some 10 ms of load to settle (launches right after an
     # idle spell run 3-5 % slow), and the whole-step figure below should be the settled one a training job sees.
     xd, ad, bd, cd = (t.detach() for t in leaves)
     with torch.no_grad():
-        _, _, ckpt, stride = hip_scan.scan_forward(xd, ad, bd, cd, out_dtype=out_dtype,
-                                                   tune=args.tune_fwd, bwd_tune=args.tune_bwd)
+        _, _, ckpt, stride = hip_scan.scan_forward(xd, ad, bd, cd, out_dtype=out_dtype)
         detached = [tuple(t.detach() for t in ops) + (gy,) for ops, gy in sets]
 
         def fwd_once():
             xs, as_, bs, cs, _ = detached[turn[0] % n_sets]
             turn[0] += 1
-            hip_scan.scan_forward(xs, as_, bs, cs, out_dtype=out_dtype, tune=args.tune_fwd, bwd_tune=args.tune_bwd)
+            hip_scan.scan_forward(xs, as_, bs, cs, out_dtype=out_dtype)
 
         def bwd_once():
             xs, as_, bs, cs, gy = detached[turn[0] % n_sets]
             turn[0] += 1
-            hip_scan.scan_backward(xs, as_, bs, cs, gy, ckpt=ckpt, ckpt_stride=stride, tune=args.tune_bwd)
+            hip_scan.scan_backward(xs, as_, bs, cs, gy, ckpt=ckpt, ckpt_stride=stride)
 
         fwd_ms = event_time_ms(torch, fwd_once, args.steps, args.warmup)
         bwd_ms = event_time_ms(torch, bwd_once, args.steps, args.warmup)
@@ -205,8 +205,8 @@ def main() -> int:
 
     status = hip_scan.workspace_status()
     align = hip_scan._align_elems([xd, ad, bd, cd, dy], D)   # what the timed launches were planned with
-    plan_b = hip_scan.make_plan(B, L, D, dtype, out_dtype, _lib.QSSM_BACKWARD, align, stride, args.tune_bwd)
-    plan_f = hip_scan.make_plan(B, L, D, dtype, out_dtype, _lib.QSSM_FORWARD, align, stride, args.tune_fwd)
+    plan_b = hip_scan.make_plan(B, L, D, dtype, out_dtype, _lib.QSSM_BACKWARD, align, stride)
+    plan_f = hip_scan.make_plan(B, L, D, dtype, out_dtype, _lib.QSSM_FORWARD, align, stride)
 
     traffic = None
     traffic_file = ROOT / "profiles" / f"scan_bwd_{args.workload}_traffic.json"

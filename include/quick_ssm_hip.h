@@ -106,16 +106,23 @@ QSSM_API const char* qssm_error_string(void);
  *                 every base address expressed in elements, over all tensors of the launch.
  *   ckpt_stride : 0 lets the forward plan pick; a backward plan (and a forward plan that must
  *                 match one) passes the stride the saved states were written with.
- *   tune        : 0 = automatic; otherwise bit fields override single choices for sweeps, a zero field
- *                 keeping the automatic one: (g_log2 + 1) | steps << 8 | max vec << 16 |
- *                 threads code << 24 (1: 256, 2: 512, 3: 1024) | (log2(cluster) + 1) << 28.
  * Stands in for the grid/block arithmetic of block_scan_forward_3d
  * (quick_ssm/triton_forwards.py:157-167) and block_scan_backward_3d
  * (quick_ssm/triton_backwards.py:195-204).
  */
 QSSM_API int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int32_t out_dtype,
-                   int32_t direction, int32_t align_elems, int32_t ckpt_stride, int32_t tune,
-                   qssm_plan* plan);
+                   int32_t direction, int32_t align_elems, int32_t ckpt_stride, qssm_plan* plan);
+
+/*
+ * qssm_plan_scan with single choices of the planner overridden.  For tests (which force every launch geometry
+ * through the same inputs) and for geometry sweeps; a binding of the reference has no use for it.
+ *   tune : bit fields, a zero field keeping the automatic choice: (g_log2 + 1) | steps << 8 | max vec << 16 |
+ *          threads code << 24 (1: 256, 2: 512, 3: 1024) | (log2(cluster) + 1) << 28.  tune = 0 is qssm_plan_scan.
+ * No counterpart in the reference.
+ */
+QSSM_API int qssm_plan_scan_tuned(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int32_t out_dtype,
+                         int32_t direction, int32_t align_elems, int32_t ckpt_stride, int32_t tune,
+                         qssm_plan* plan);
 
 /*
  * Two device buffers accompany every launch, both owned by the caller and both zero-filled
@@ -123,9 +130,10 @@ QSSM_API int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, i
  *
  *   control    status word, a launch count and one ticket counter per chain (plan.control_bytes).
  *              A launch needs the status word and the ticket counters zero on entry and leaves them
- *              zero, except that the status word becomes nonzero if a tile gave up waiting for a
- *              neighbour (the outputs of that launch are then poisoned with NaN and the buffer
- *              must be zero-filled again).
+ *              zero, except that the status word becomes 1 if a tile gave up waiting for a neighbour
+ *              (outputs downstream of it are NaN), and 2 if a ticket counter was not zero on entry
+ *              (every output of the launch is NaN).  Either way the results are invalid and both
+ *              buffers must be zero-filled again before the next launch.
  *   workspace  the words tiles hand to each other (plan.workspace_bytes; may be 0).  Words are
  *              tagged with the launch's epoch, so nothing has to be cleared between launches:
  *              zero-fill it once, and again before an epoch value would be reused.
@@ -145,6 +153,11 @@ QSSM_API int qssm_zero_fill(void* buffer, uint64_t bytes, void* stream);
 /* Read back the status word of a control block (synchronises `stream`).  0 = every launch since
  * the last zero-fill completed. */
 QSSM_API int qssm_control_status(const void* control, void* stream, int32_t* status);
+
+/* Enqueue a copy of the status word into `host_status` (pinned host memory) on `stream`, without waiting:
+ * the word is sticky until the control block is zero-filled, so a later look at `host_status` sees any failure
+ * of a launch ordered before the copy.  What a training loop polls instead of synchronising. */
+QSSM_API int qssm_control_status_async(const void* control, int32_t* host_status, void* stream);
 
 /*
  * Forward scan: one pass that reads x, a, b, c once and writes y once.
@@ -273,6 +286,52 @@ QSSM_API int qssm_scan_backward_carry(const qssm_plan* plan,
                              void* control, uint64_t control_size,
                              void* workspace, uint64_t workspace_bytes, uint32_t epoch,
                              void* stream);
+
+/*
+ * The same two launches with their arguments in one block: a binding that keeps such a block per shape only
+ * patches the pointers between calls, which matters where launches are small enough for the host side of a call
+ * to bound the step (the reference's copy task: B=32, L=64, 12 layers).  Fields as the arguments of
+ * qssm_scan_forward_carry / qssm_scan_backward_carry of the same names.
+ */
+typedef struct qssm_forward_call {
+  const qssm_plan* plan;
+  const void *x, *a, *b, *c;
+  void* y;
+  float* h_out;
+  float* ckpt;
+  const float* h_init;
+  float* h_final;
+  qssm_strides sx, sa, sb, sc, sy, sh;
+  void* control;
+  uint64_t control_size;
+  void* workspace;
+  uint64_t workspace_bytes;
+  uint32_t epoch;
+  uint32_t reserved;
+  void* stream;
+} qssm_forward_call;
+
+typedef struct qssm_backward_call {
+  const qssm_plan* plan;
+  const void *x, *a, *b, *c, *dy;
+  const float* h;
+  const float* ckpt;
+  const float* h_init;
+  const float* dh_final;
+  float* dh_init;
+  void *dx, *da, *db, *dc;
+  qssm_strides sx, sa, sb, sc, sdy, sh, sdx, sda, sdb, sdc;
+  void* control;
+  uint64_t control_size;
+  void* workspace;
+  uint64_t workspace_bytes;
+  uint32_t epoch;
+  uint32_t reserved;
+  void* stream;
+} qssm_backward_call;
+
+QSSM_API int qssm_scan_forward_call(const qssm_forward_call* call);
+QSSM_API int qssm_scan_backward_call(const qssm_backward_call* call);
 
 /*
  * Gate prologue of the SSM layer: the five projection outputs [rows, S] (row strides ld_* in elements,

@@ -24,13 +24,17 @@ EXPORTED_SYMBOLS = (
     "qssm_version",
     "qssm_error_string",
     "qssm_plan_scan",
+    "qssm_plan_scan_tuned",
     "qssm_zero_fill",
     "qssm_control_status",
+    "qssm_control_status_async",
     "qssm_scan_forward",
     "qssm_scan_backward",
     "qssm_scan_forward_carry",
     "qssm_scan_backward_carry",
     "qssm_scan_forward_static",
+    "qssm_scan_forward_call",
+    "qssm_scan_backward_call",
     "qssm_gates_forward",
     "qssm_gates_backward",
     "qssm_rmsnorm_forward",
@@ -78,6 +82,33 @@ class Strides(ctypes.Structure):
     _fields_ = [("b", ctypes.c_int64), ("l", ctypes.c_int64)]
 
 
+class ForwardCall(ctypes.Structure):
+    """Mirror of `qssm_forward_call`."""
+
+    _fields_ = (
+        [("plan", ctypes.POINTER(Plan))]
+        + [(n, ctypes.c_void_p) for n in ("x", "a", "b", "c", "y", "h_out", "ckpt", "h_init", "h_final")]
+        + [(n, Strides) for n in ("sx", "sa", "sb", "sc", "sy", "sh")]
+        + [("control", ctypes.c_void_p), ("control_size", ctypes.c_uint64), ("workspace", ctypes.c_void_p),
+           ("workspace_bytes", ctypes.c_uint64), ("epoch", ctypes.c_uint32), ("reserved", ctypes.c_uint32),
+           ("stream", ctypes.c_void_p)]
+    )
+
+
+class BackwardCall(ctypes.Structure):
+    """Mirror of `qssm_backward_call`."""
+
+    _fields_ = (
+        [("plan", ctypes.POINTER(Plan))]
+        + [(n, ctypes.c_void_p) for n in ("x", "a", "b", "c", "dy", "h", "ckpt", "h_init", "dh_final", "dh_init",
+                                          "dx", "da", "db", "dc")]
+        + [(n, Strides) for n in ("sx", "sa", "sb", "sc", "sdy", "sh", "sdx", "sda", "sdb", "sdc")]
+        + [("control", ctypes.c_void_p), ("control_size", ctypes.c_uint64), ("workspace", ctypes.c_void_p),
+           ("workspace_bytes", ctypes.c_uint64), ("epoch", ctypes.c_uint32), ("reserved", ctypes.c_uint32),
+           ("stream", ctypes.c_void_p)]
+    )
+
+
 class QssmError(RuntimeError):
     def __init__(self, code: int, message: str):
         super().__init__(f"libquick_ssm_hip: {message} (code {code})")
@@ -95,7 +126,15 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.qssm_error_string.restype = ctypes.c_char_p
     lib.qssm_error_string.argtypes = []
     lib.qssm_plan_scan.restype = ctypes.c_int
-    lib.qssm_plan_scan.argtypes = [i32] * 9 + [ctypes.POINTER(Plan)]
+    lib.qssm_plan_scan.argtypes = [i32] * 8 + [ctypes.POINTER(Plan)]
+    lib.qssm_plan_scan_tuned.restype = ctypes.c_int
+    lib.qssm_plan_scan_tuned.argtypes = [i32] * 9 + [ctypes.POINTER(Plan)]
+    lib.qssm_control_status_async.restype = ctypes.c_int
+    lib.qssm_control_status_async.argtypes = [vp, vp, vp]
+    lib.qssm_scan_forward_call.restype = ctypes.c_int
+    lib.qssm_scan_forward_call.argtypes = [vp]
+    lib.qssm_scan_backward_call.restype = ctypes.c_int
+    lib.qssm_scan_backward_call.argtypes = [vp]
     lib.qssm_zero_fill.restype = ctypes.c_int
     lib.qssm_zero_fill.argtypes = [vp, u64, vp]
     lib.qssm_control_status.restype = ctypes.c_int

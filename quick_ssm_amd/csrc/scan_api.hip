@@ -186,7 +186,12 @@ int qssm_version(void) { return QSSM_VERSION; }
 const char* qssm_error_string(void) { return g_err; }
 
 int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int32_t out_dtype, int32_t direction,
-                   int32_t align_elems, int32_t ckpt_stride, int32_t tune, qssm_plan* plan) {
+                   int32_t align_elems, int32_t ckpt_stride, qssm_plan* plan) {
+  return qssm_plan_scan_tuned(B, L, D, in_dtype, out_dtype, direction, align_elems, ckpt_stride, 0, plan);
+}
+
+int qssm_plan_scan_tuned(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int32_t out_dtype, int32_t direction,
+                         int32_t align_elems, int32_t ckpt_stride, int32_t tune, qssm_plan* plan) {
   if (plan == nullptr) return fail(QSSM_EINVAL, "plan is NULL");
   if (B < 0 || L < 0 || D < 0) return fail(QSSM_EINVAL, "negative dimension");
   if (direction != QSSM_FORWARD && direction != QSSM_BACKWARD) return fail(QSSM_EINVAL, "bad direction");
@@ -356,6 +361,27 @@ int qssm_control_status(const void* control, void* stream, int32_t* status) {
   if (e != hipSuccess) return hip_fail(e, "hipMemcpyAsync(status)");
   e = hipStreamSynchronize((hipStream_t)stream);
   return e == hipSuccess ? 0 : hip_fail(e, "hipStreamSynchronize");
+}
+
+int qssm_control_status_async(const void* control, int32_t* host_status, void* stream) {
+  if (control == nullptr || host_status == nullptr) return fail(QSSM_EINVAL, "NULL argument");
+  hipError_t e = hipMemcpyAsync(host_status, control, sizeof(int32_t), hipMemcpyDeviceToHost, (hipStream_t)stream);
+  return e == hipSuccess ? 0 : hip_fail(e, "hipMemcpyAsync(status)");
+}
+
+int qssm_scan_forward_call(const qssm_forward_call* k) {
+  if (k == nullptr) return fail(QSSM_EINVAL, "call is NULL");
+  return forward_launch(k->plan, k->x, k->sx, k->a, k->sa, k->b, k->sb, k->c, k->sc, k->y, k->sy, k->h_out, k->sh,
+                        k->ckpt, k->h_init, k->h_final, k->control, k->control_size, k->workspace,
+                        k->workspace_bytes, k->epoch, kCountWrapAt, k->stream);
+}
+
+int qssm_scan_backward_call(const qssm_backward_call* k) {
+  if (k == nullptr) return fail(QSSM_EINVAL, "call is NULL");
+  return qssm_scan_backward_carry(k->plan, k->x, k->sx, k->a, k->sa, k->b, k->sb, k->c, k->sc, k->dy, k->sdy, k->h,
+                                  k->sh, k->ckpt, k->h_init, k->dh_final, k->dh_init, k->dx, k->sdx, k->da, k->sda,
+                                  k->db, k->sdb, k->dc, k->sdc, k->control, k->control_size, k->workspace,
+                                  k->workspace_bytes, k->epoch, k->stream);
 }
 
 int qssm_scan_forward(const qssm_plan* plan, const void* x, qssm_strides sx, const void* a, qssm_strides sa,

@@ -62,8 +62,31 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
     if (tid == 0) *sSeg = (int)claim_ticket(g.tickets, chain, g.n_seg);
     __syncthreads();
     const int tk = __builtin_amdgcn_readfirstlane(*sSeg);
-    if ((unsigned)tk >= (unsigned)g.n_seg) {  // the control block was not zero on entry
+    if ((unsigned)tk >= (unsigned)g.n_seg) {
+      // The control block was not zero on entry: no tile can be claimed in order.  Every workgroup then poisons
+      // the tile its index names (the grid has one workgroup per tile), so that the caller never reads memory
+      // nobody wrote, and reports it.
       if (tid == 0) raise_status(g.status, 2);
+      const int pseg = blockIdx.x / g.n_chains, pbi = chain / g.n_strips, pstrip = chain - pbi * g.n_strips;
+      const int pd = pstrip * cols + (tid & (G - 1)) * VEC;
+      float nanv[VEC];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) nanv[v] = __uint_as_float(0x7fc00000u);
+      for (int i = 0; i < T; ++i) {
+        const int t = pseg * g.seg_len + (tid >> g.g_log2) * T + i;
+        if (pd < g.D && t < g.L) {
+          if (p.dx != nullptr)
+            store_stream<Tin, VEC>((char*)p.dx + ((int64_t)pbi * p.dx_sb + (int64_t)t * p.dx_sl + pd) * (int64_t)sizeof(Tin), 0u, nanv);
+          if (p.da != nullptr)
+            store_stream<Tin, VEC>((char*)p.da + ((int64_t)pbi * p.da_sb + (int64_t)t * p.da_sl + pd) * (int64_t)sizeof(Tin), 0u, nanv);
+          if (p.db != nullptr)
+            store_stream<Tin, VEC>((char*)p.db + ((int64_t)pbi * p.db_sb + (int64_t)t * p.db_sl + pd) * (int64_t)sizeof(Tin), 0u, nanv);
+          if (p.dc != nullptr)
+            store_stream<Tin, VEC>((char*)p.dc + ((int64_t)pbi * p.dc_sb + (int64_t)t * p.dc_sl + pd) * (int64_t)sizeof(Tin), 0u, nanv);
+        }
+      }
+      if (p.dh_init != nullptr && pseg == 0 && (tid >> g.g_log2) == 0 && pd < g.D)
+        store_stream<float, VEC>((char*)p.dh_init + ((int64_t)pbi * g.D + pd) * (int64_t)sizeof(float), 0u, nanv);
       return;
     }
     seg = g.n_seg - 1 - tk;

@@ -51,8 +51,29 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
     if (tid == 0) *sSeg = (int)claim_ticket(g.tickets, chain, g.n_seg);
     __syncthreads();
     seg = __builtin_amdgcn_readfirstlane(*sSeg);
-    if ((unsigned)seg >= (unsigned)g.n_seg) {  // the control block was not zero on entry
+    if ((unsigned)seg >= (unsigned)g.n_seg) {
+      // The control block was not zero on entry: no tile can be claimed in order.  Every workgroup then poisons
+      // the tile its index names (the grid has one workgroup per tile), so that the caller never reads memory
+      // nobody wrote, and reports it.
       if (tid == 0) raise_status(g.status, 2);
+      const int pseg = blockIdx.x / g.n_chains, pbi = chain / g.n_strips, pstrip = chain - pbi * g.n_strips;
+      const int pd = pstrip * cols + (tid & (G - 1)) * VEC;
+      float nanv[VEC];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) nanv[v] = __uint_as_float(0x7fc00000u);
+      for (int i = 0; i < T; ++i) {
+        const int t = pseg * g.seg_len + (tid >> g.g_log2) * T + i;
+        if (pd < g.D && t < g.L) {
+          if (p.y != nullptr)
+            store_stream<Tout, VEC>((char*)p.y + ((int64_t)pbi * p.y_sb + (int64_t)t * p.y_sl + pd) * (int64_t)sizeof(Tout), 0u, nanv);
+          if (p.h_out != nullptr)
+            store_stream<float, VEC>((char*)p.h_out + ((int64_t)pbi * p.h_sb + (int64_t)t * p.h_sl + pd) * (int64_t)sizeof(float), 0u, nanv);
+          if (p.ckpt != nullptr && t % g.ckpt_stride == 0)
+            store_stream<float, VEC>((char*)p.ckpt + (((int64_t)pbi * g.n_ckpt + t / g.ckpt_stride) * g.D + pd) * (int64_t)sizeof(float), 0u, nanv);
+        }
+      }
+      if (p.h_final != nullptr && pseg == g.n_seg - 1 && (tid >> g.g_log2) == 0 && pd < g.D)
+        store_stream<float, VEC>((char*)p.h_final + ((int64_t)pbi * g.D + pd) * (int64_t)sizeof(float), 0u, nanv);
       return;
     }
   }

@@ -9,13 +9,14 @@ direction.
 from __future__ import annotations
 
 import ctypes
+import os
 import threading
-from typing import Dict, Optional, Sequence, Tuple
+from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
 from . import _lib
-from ._lib import Plan, Strides
+from ._lib import BackwardCall, ForwardCall, Plan, Strides
 
 Tensor = torch.Tensor
 
@@ -31,18 +32,67 @@ _ws_lock = threading.Lock()
 _EPOCH_MAX = 0xFFFFFFFF
 
 
+class ScanLaunchError(RuntimeError):
+    """A scan launch reported failure through its control block's status word.
+
+    status 1: a tile gave up waiting for a neighbour's word (about a second); outputs downstream of it are NaN.
+    status 2: a ticket counter was not zero when the launch started; every output of the launch is NaN.
+    By the time this is raised the control block and workspace have been zero-filled again, so the next launch
+    on the stream starts clean; results of launches since the last check must be discarded.
+    """
+
+    def __init__(self, status: int, where: str):
+        super().__init__(
+            f"quick_ssm_amd: a scan launch on {where} failed with status {status} "
+            f"({'a tile gave up waiting for a neighbour' if status == 1 else 'the control block was not zero on entry' if status == 2 else 'both kinds of failure'}); "
+            "its outputs are NaN. Control block and workspace have been reset; repeat the step.")
+        self.status = status
+
+
+def _env_int(name: str, default: int) -> int:
+    try:
+        return int(os.environ.get(name, default))
+    except ValueError:
+        return default
+
+
+# Every `_check_every`-th launch on a pair of buffers is followed by an asynchronous copy of the status word to
+# pinned host memory, looked at (without waiting) before each later launch: a failed launch is reported within two
+# such periods.  QSSM_CHECK_STATUS=1 checks behind every launch, 0 never; set_status_check_period() at run time.
+_check_every = _env_int("QSSM_CHECK_STATUS", 64)
+
+
+def set_status_check_period(launches: int) -> int:
+    """Look at the status word every `launches`-th launch (0: never).  Returns the old period."""
+    global _check_every
+    old, _check_every = _check_every, max(0, int(launches))
+    return old
+
+
 class _Buffers:
-    """Per (device, stream, who numbers the launches): control block, workspace, and the host's launch count."""
+    """Per (device, stream, who numbers the launches): control block, workspace, the host's launch count, and the
+    pinned word the status is copied to."""
 
-    __slots__ = ("control", "workspace", "epoch")
+    __slots__ = ("control", "workspace", "epoch", "ctl_ptr", "ctl_size", "ws_ptr", "ws_size", "captured",
+                 "pinned", "seen", "since_check", "device", "where")
 
-    def __init__(self):
+    def __init__(self, device: torch.device, where: str):
         self.control: Optional[Tensor] = None
         self.workspace: Optional[Tensor] = None
         self.epoch = 0
+        self.ctl_ptr = self.ctl_size = self.ws_ptr = self.ws_size = 0
+        self.captured = False          # a graph holds these addresses: never free or move them
+        self.pinned = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+        self.seen = ctypes.c_int32.from_address(self.pinned.data_ptr())
+        self.since_check = 0
+        self.device = device
+        self.where = where
 
 
 _buffers: Dict[Tuple[int, int, bool], _Buffers] = {}
+# Buffers a recorded graph still points to, after they have been replaced by larger ones or dropped by
+# reset_workspaces(): kept alive until the process ends, because replaying that graph writes to them.
+_retired: List[Tensor] = []
 
 
 def kernel_dtypes(in_dtypes: Sequence[torch.dtype], out_dtype: torch.dtype) -> Tuple[torch.dtype, torch.dtype]:
@@ -53,7 +103,8 @@ def kernel_dtypes(in_dtypes: Sequence[torch.dtype], out_dtype: torch.dtype) -> T
     """
     common = in_dtypes[0]
     for dt in in_dtypes[1:]:
-        common = torch.promote_types(common, dt)
+        if dt != common:
+            common = torch.promote_types(common, dt)
     if common not in _DTYPE_CODE:
         common = torch.float32
     k_out = out_dtype if out_dtype in _BUILT_OUT[common] else torch.float32
@@ -62,11 +113,7 @@ def kernel_dtypes(in_dtypes: Sequence[torch.dtype], out_dtype: torch.dtype) -> T
 
 def _unit_inner(t: Tensor) -> Tensor:
     """A view or copy of `t` whose last axis is contiguous."""
-    if t.size(-1) > 1 and t.stride(-1) != 1:
-        return t.contiguous()
-    if t.size(-1) == 1 and t.stride(-1) != 1:
-        return t.contiguous()
-    return t
+    return t if t.stride(2) == 1 else t.contiguous()
 
 
 def _strides(t: Optional[Tensor]) -> Strides:
@@ -81,47 +128,102 @@ def _ptr(t: Optional[Tensor]) -> Optional[int]:
 
 def _align_elems(tensors: Sequence[Optional[Tensor]], D: int) -> int:
     """Largest v in (8, 4, 2, 1) such that D, every stride and every base address (in elements) divide by v."""
-    for v in (8, 4, 2):
-        ok = D % v == 0
-        for t in tensors:
-            if not ok:
-                break
-            if t is None:
-                continue
-            es = t.element_size()
-            ok = t.data_ptr() % (es * v) == 0 and t.stride(0) % v == 0 and t.stride(1) % v == 0
-        if ok:
-            return v
-    return 1
+    bits = D
+    for t in tensors:
+        if t is None:
+            continue
+        es = t.element_size()
+        ptr = t.data_ptr()
+        if ptr % es:
+            return 1
+        bits |= (ptr // es) | t.stride(0) | t.stride(1)
+    low = bits & -bits
+    return 8 if low == 0 or low > 8 else low
 
 
-_device_counted_depth = 0  # contexts open right now, in any thread (guarded by _ws_lock)
+# (device index, stream handle) -> how many `device_counted_launches` contexts are open on it
+_device_counted: Dict[Tuple[int, int], int] = {}
+
+
+def _raw_stream(dev_index: int) -> int:
+    return torch._C._cuda_getCurrentRawStream(dev_index)
 
 
 class device_counted_launches:
-    """Context manager: scan launches made while it is open, from any thread (autograd runs the backward on its
-    own), number themselves in their control block (epoch argument 0), as launches recorded into a graph do, and use
-    the buffers kept for such launches.
+    """Context manager: scan launches made on the stream that is current when it is entered, while it is open and
+    from any thread (autograd runs the backward on its own, on the forward's stream), number themselves in their
+    control block (epoch argument 0), as launches recorded into a graph do, and use the buffers kept for such
+    launches.  Launches on other streams or devices are not affected.
 
     Launches being recorded into a graph do this by themselves, but cannot allocate: run the work once inside this
     context, on the stream that will capture, and the control block and workspace exist (large enough) when the
-    capture starts.
+    capture starts.  Buffers a capture has used are never freed: if a later launch needs larger ones, new buffers
+    take their place for new launches and the old ones stay alive for the graph that points to them.  Two graphs
+    recorded on one stream share their buffers: replay them on that stream, one at a time.
     """
 
     def __enter__(self):
-        global _device_counted_depth
+        index = torch.cuda.current_device()
+        self._key = (index, _raw_stream(index))
         with _ws_lock:
-            _device_counted_depth += 1
+            _device_counted[self._key] = _device_counted.get(self._key, 0) + 1
         return self
 
     def __exit__(self, *exc):
-        global _device_counted_depth
         with _ws_lock:
-            _device_counted_depth -= 1
+            left = _device_counted.get(self._key, 0) - 1
+            if left > 0:
+                _device_counted[self._key] = left
+            else:
+                _device_counted.pop(self._key, None)
         return False
 
 
-def _launch_buffers(device: torch.device, stream: int, plan: Plan) -> Tuple[Tensor, Tensor, int]:
+def _grow_buffers(key: Tuple[int, int, bool], device: torch.device, need_c: int, need_w: int, capturing: bool) -> _Buffers:
+    """Slow path of `_launch_buffers`: first use of a (device, stream), a larger shape, or a used-up numbering."""
+    with _ws_lock:
+        buf = _buffers.get(key)
+        grow_c = buf is None or buf.control is None or buf.ctl_size < need_c
+        grow_w = grow_c or buf.workspace is None or buf.ws_size < need_w or buf.epoch >= _EPOCH_MAX
+        if capturing and grow_w:   # before anything is allocated: an allocation would spoil the recording
+            raise RuntimeError(
+                "quick_ssm_amd: a scan launch being recorded into a graph cannot allocate its control block and "
+                "workspace; run the same work once inside `hip_scan.device_counted_launches()` on this stream first")
+        if buf is None:
+            buf = _Buffers(device, f"device {key[0]}, stream {key[1]:#x}")
+        if buf.captured and grow_w:
+            # a recorded graph points at the old pair: keep it alive and untouched, new launches get a new pair
+            _retired.extend(t for t in (buf.control, buf.workspace) if t is not None)
+            buf.captured = False
+            grow_c = True
+        if grow_c:
+            # a new control block restarts the device-side count: the workspace must not keep words of the old numbering
+            buf.control = torch.zeros(max(1 << 16, 1 << (need_c - 1).bit_length()), dtype=torch.uint8, device=device)
+            buf.ctl_ptr, buf.ctl_size = buf.control.data_ptr(), buf.control.numel()
+        if grow_w:
+            buf.workspace = torch.zeros(max(1 << 20, 1 << (need_w - 1).bit_length()), dtype=torch.uint8, device=device)
+            buf.ws_ptr, buf.ws_size = buf.workspace.data_ptr(), buf.workspace.numel()
+            buf.epoch = 0
+        _buffers[key] = buf
+        return buf
+
+
+def _recover(buf: _Buffers, stream: int) -> int:
+    """Zero-fill a failed pair of buffers on `stream`, forget the host's numbering, and return the status seen."""
+    lib = _lib.load()
+    with torch.cuda.device(buf.device):
+        _lib.check(lib.qssm_zero_fill(buf.ctl_ptr, buf.ctl_size, stream))
+        _lib.check(lib.qssm_zero_fill(buf.ws_ptr, buf.ws_size, stream))
+        out = ctypes.c_int32(0)
+        _lib.check(lib.qssm_control_status(buf.ctl_ptr, stream, ctypes.byref(out)))   # waits: copies in flight have landed
+    status = int(buf.seen.value)
+    buf.seen.value = 0
+    buf.epoch = 0
+    buf.since_check = 0
+    return status
+
+
+def _launch_buffers(device: torch.device, dev_index: int, stream: int, need_c: int, need_w: int) -> Tuple[_Buffers, int, bool]:
     """Control block, workspace and epoch argument for the next launch on (device, stream).
 
     Both buffers are zero-filled when they are allocated (torch.zeros runs a fill kernel on the
@@ -131,55 +233,60 @@ def _launch_buffers(device: torch.device, stream: int, plan: Plan) -> Tuple[Tens
     graph (and those inside `device_counted_launches`) use a pair of buffers of their own and are
     numbered in the control block itself (epoch argument 0), so that replays number themselves, at
     the price of a one-lane counting kernel behind each launch.  A workspace that has to grow, or
-    whose 32-bit host numbering is used up, is replaced by a fresh zeroed one.
+    whose 32-bit host numbering is used up, is replaced by a fresh zeroed one.  A status word that an
+    earlier check found nonzero raises ScanLaunchError here, after the buffers have been reset.
     """
-    capturing = bool(torch.cuda.is_current_stream_capturing())
-    on_device = capturing or _device_counted_depth > 0
-    key = (device.index if device.index is not None else torch.cuda.current_device(), stream, on_device)
-    with _ws_lock:
-        buf = _buffers.get(key)
-        if buf is None:
-            buf = _Buffers()
-        need_c, need_w = int(plan.control_bytes), max(int(plan.workspace_bytes), 256)
-        grow_c = buf.control is None or buf.control.numel() < need_c
-        grow_w = grow_c or buf.workspace is None or buf.workspace.numel() < need_w or buf.epoch >= _EPOCH_MAX
-        if capturing and grow_w:
-            raise RuntimeError(
-                "quick_ssm_amd: a scan launch being recorded into a graph cannot allocate its control block and "
-                "workspace; run the same work once inside `hip_scan.device_counted_launches()` on this stream first")
-        _buffers[key] = buf
-        if grow_c:
-            # a new control block restarts the device-side count: the workspace must not keep words of the old numbering
-            buf.control = torch.zeros(max(1 << 16, 1 << (need_c - 1).bit_length()), dtype=torch.uint8, device=device)
-        if grow_w:
-            buf.workspace = torch.zeros(max(1 << 20, 1 << (need_w - 1).bit_length()), dtype=torch.uint8, device=device)
-            buf.epoch = 0
-        if on_device:
-            return buf.control, buf.workspace, 0
-        buf.epoch += 1
-        return buf.control, buf.workspace, buf.epoch
+    capturing = torch._C._cuda_isCurrentStreamCapturing()
+    on_device = capturing or ((dev_index, stream) in _device_counted)
+    key = (dev_index, stream, on_device)
+    buf = _buffers.get(key)
+    if buf is None or buf.ctl_size < need_c or buf.ws_size < need_w or buf.epoch >= _EPOCH_MAX:
+        buf = _grow_buffers(key, device, need_c, max(need_w, 256), capturing)
+    if buf.seen.value != 0 and not capturing:
+        raise ScanLaunchError(_recover(buf, stream), buf.where)
+    if capturing:
+        buf.captured = True
+    if on_device:
+        return buf, 0, capturing
+    buf.epoch += 1
+    return buf, buf.epoch, capturing
 
 
-def workspace_status(device: Optional[torch.device] = None) -> int:
-    """Status words of the current stream's control blocks, or-ed (synchronises).  0 = all launches completed."""
+def _after_launch(buf: _Buffers, stream: int, capturing: bool) -> None:
+    """Every `_check_every`-th launch: ask for the status word, to be looked at before a later launch."""
+    if _check_every <= 0 or capturing:
+        return
+    buf.since_check += 1
+    if buf.since_check >= _check_every:
+        buf.since_check = 0
+        _lib.check(_lib.load().qssm_control_status_async(buf.ctl_ptr, buf.pinned.data_ptr(), stream))
+
+
+def workspace_status(device: Optional[torch.device] = None, all_streams: bool = False) -> int:
+    """Status words of the current stream's control blocks (of every stream of the device with `all_streams`),
+    or-ed; synchronises those streams.  0 = all launches completed."""
     device = torch.device("cuda", torch.cuda.current_device()) if device is None else device
-    stream = torch.cuda.current_stream(device).cuda_stream
     index = device.index if device.index is not None else torch.cuda.current_device()
+    stream = _raw_stream(index)
+    with _ws_lock:
+        bufs = [(k, b) for k, b in _buffers.items()
+                if k[0] == index and (all_streams or k[1] == stream) and b.control is not None]
     status = 0
-    for on_device in (False, True):
-        with _ws_lock:
-            buf = _buffers.get((index, stream, on_device))
-        if buf is None or buf.control is None:
-            continue
+    for key, buf in bufs:
         out = ctypes.c_int32(0)
-        _lib.check(_lib.load().qssm_control_status(buf.control.data_ptr(), stream, ctypes.byref(out)))
+        with torch.cuda.device(device):
+            _lib.check(_lib.load().qssm_control_status(buf.ctl_ptr, key[1], ctypes.byref(out)))
         status |= int(out.value)
     return status
 
 
 def reset_workspaces() -> None:
-    """Drop every cached buffer (the next launch allocates fresh zeroed ones)."""
+    """Drop every cached buffer (the next launch allocates fresh zeroed ones).  Buffers that a recorded graph
+    points to are not freed, but no later launch uses them: such graphs still replay, on their own old buffers."""
     with _ws_lock:
+        for buf in _buffers.values():
+            if buf.captured:
+                _retired.extend(t for t in (buf.control, buf.workspace) if t is not None)
         _buffers.clear()
 
 
@@ -188,20 +295,58 @@ _plans: Dict[tuple, Plan] = {}
 
 def make_plan(B: int, L: int, D: int, in_dtype: torch.dtype, out_dtype: torch.dtype, direction: int,
               align_elems: int, ckpt_stride: int = 0, tune: int = 0) -> Plan:
-    """Launch geometry for a shape (qssm_plan_scan).  Plans depend on nothing but the arguments, so they are
-    kept: small problems are bound by the host side of a launch.  Callers must not modify the result."""
+    """Launch geometry for a shape (qssm_plan_scan; qssm_plan_scan_tuned when a test or sweep overrides single
+    choices with `tune`).  Plans depend on nothing but the arguments, so they are kept: small problems are bound by
+    the host side of a launch.  Callers must not modify the result."""
     key = (B, L, D, in_dtype, out_dtype, direction, align_elems, ckpt_stride, tune)
     plan = _plans.get(key)
     if plan is None:
         plan = Plan()
-        _lib.check(
-            _lib.load().qssm_plan_scan(B, L, D, _DTYPE_CODE[in_dtype], _DTYPE_CODE[out_dtype], direction,
-                                       align_elems, ckpt_stride, tune, ctypes.byref(plan))
-        )
+        lib = _lib.load()
+        if tune:
+            rc = lib.qssm_plan_scan_tuned(B, L, D, _DTYPE_CODE[in_dtype], _DTYPE_CODE[out_dtype], direction,
+                                          align_elems, ckpt_stride, tune, ctypes.byref(plan))
+        else:
+            rc = lib.qssm_plan_scan(B, L, D, _DTYPE_CODE[in_dtype], _DTYPE_CODE[out_dtype], direction,
+                                    align_elems, ckpt_stride, ctypes.byref(plan))
+        _lib.check(rc)
         if len(_plans) >= 4096:
             _plans.clear()
         _plans[key] = plan
     return plan
+
+
+class _Launch:
+    """A ready-made argument block for one (direction, shape, storage, alignment, geometry): the plan, what the
+    host needs from it as plain ints, and the ctypes block whose pointers a call patches."""
+
+    __slots__ = ("plan", "call", "call_ref", "need_c", "need_w", "n_ckpt", "ckpt_stride", "strides")
+
+    def __init__(self, plan: Plan, call):
+        self.plan = plan
+        self.call = call
+        self.call_ref = ctypes.byref(call)
+        call.plan = ctypes.pointer(plan)
+        self.need_c = int(plan.control_bytes)
+        self.need_w = int(plan.workspace_bytes)
+        self.n_ckpt = int(plan.n_ckpt)
+        self.ckpt_stride = int(plan.ckpt_stride)
+        self.strides = None   # the stride tuples the block's stride fields were last filled from
+
+
+_tls = threading.local()   # argument blocks are patched in place, so every thread keeps its own
+
+
+def _launch_entry(key: tuple, make) -> _Launch:
+    cache = getattr(_tls, "launches", None)
+    if cache is None:
+        cache = _tls.launches = {}
+    entry = cache.get(key)
+    if entry is None:
+        if len(cache) >= 1024:
+            cache.clear()
+        entry = cache[key] = make()
+    return entry
 
 
 def _require_gpu(*tensors: Tensor) -> torch.device:
@@ -223,6 +368,9 @@ def _check_state(t: Optional[Tensor], B: int, D: int, dev: torch.device, name: s
                          f"got {t.dtype} {tuple(t.shape)} on {t.device}")
 
 
+_NO_STRIDE = (0, 0, 0)
+
+
 def scan_forward(
     x: Tensor, a: Tensor, b: Tensor, c: Optional[Tensor], *,
     out_dtype: torch.dtype,
@@ -241,14 +389,14 @@ def scan_forward(
     `want_ckpt` (what the backward rebuilds h from).  `h_init` (fp32 [B, D], contiguous) is the
     state before the first step instead of zero; `h_final` (same layout) receives h(L-1).
     """
-    ops = [x, a, b] + ([c] if c is not None else [])
-    dev = _require_gpu(*ops)
+    dev = _require_gpu(x, a, b) if c is None else _require_gpu(x, a, b, c)
     B, L, D = x.shape
     in_dtype = x.dtype
     y = torch.empty((B, L, D), dtype=out_dtype, device=dev) if want_y else None
     h = torch.empty((B, L, D), dtype=torch.float32, device=dev) if want_h else None
-    _check_state(h_init, B, D, dev, "h_init")
-    _check_state(h_final, B, D, dev, "h_final")
+    if h_init is not None or h_final is not None:
+        _check_state(h_init, B, D, dev, "h_init")
+        _check_state(h_final, B, D, dev, "h_final")
     if B == 0 or L == 0 or D == 0:
         if h_final is not None:  # nothing happened to the state
             h_final.copy_(h_init) if h_init is not None else h_final.zero_()
@@ -256,29 +404,51 @@ def scan_forward(
 
     x, a, b = _unit_inner(x), _unit_inner(a), _unit_inner(b)
     c = _unit_inner(c) if c is not None else None
-    align = _align_elems([x, a, b, c, y, h], D)
+    tensors = (x, a, b, c, y, h)
+    strides = tuple(_NO_STRIDE if t is None else t.stride() for t in tensors)
+    ptrs = [0 if t is None else t.data_ptr() for t in tensors]
+    align = _align_elems(tensors, D)
 
-    ckpt_stride = 0
-    if want_ckpt:
-        # The backward decides how far apart the saved states may be; the forward follows.
-        ckpt_stride = make_plan(B, L, D, in_dtype, out_dtype, _lib.QSSM_BACKWARD, align, 0, bwd_tune).seg_len
-    plan = make_plan(B, L, D, in_dtype, out_dtype, _lib.QSSM_FORWARD, align, ckpt_stride, tune)
-    ckpt = None
-    if want_ckpt:
-        ckpt = torch.empty((B, plan.n_ckpt, D), dtype=torch.float32, device=dev)
+    def make() -> _Launch:
+        stride = 0
+        if want_ckpt:
+            # The backward decides how far apart the saved states may be; the forward follows.
+            stride = make_plan(B, L, D, in_dtype, out_dtype, _lib.QSSM_BACKWARD, align, 0, bwd_tune).seg_len
+        return _Launch(make_plan(B, L, D, in_dtype, out_dtype, _lib.QSSM_FORWARD, align, stride, tune), ForwardCall())
 
-    with torch.cuda.device(dev):
-        stream = torch.cuda.current_stream(dev).cuda_stream
-        ctl, ws, epoch = _launch_buffers(dev, stream, plan)
-        _lib.check(
-            _lib.load().qssm_scan_forward_carry(
-                ctypes.byref(plan),
-                _ptr(x), _strides(x), _ptr(a), _strides(a), _ptr(b), _strides(b), _ptr(c), _strides(c),
-                _ptr(y), _strides(y), _ptr(h), _strides(h), _ptr(ckpt), _ptr(h_init), _ptr(h_final),
-                ctl.data_ptr(), ctl.numel(), ws.data_ptr(), ws.numel(), epoch, stream,
-            )
-        )
-    return y, h, ckpt, int(plan.ckpt_stride)
+    entry = _launch_entry((0, B, L, D, in_dtype, out_dtype, align, want_ckpt, tune, bwd_tune), make)
+    ckpt = torch.empty((B, entry.n_ckpt, D), dtype=torch.float32, device=dev) if want_ckpt else None
+
+    k = entry.call
+    if entry.strides != strides:
+        k.sx, k.sa, k.sb, k.sc, k.sy, k.sh = (Strides(s[0], s[1]) for s in strides)
+        entry.strides = strides
+    k.x, k.a, k.b, k.c, k.y, k.h_out = ptrs
+    k.ckpt = None if ckpt is None else ckpt.data_ptr()
+    k.h_init = None if h_init is None else h_init.data_ptr()
+    k.h_final = None if h_final is None else h_final.data_ptr()
+
+    index = dev.index
+    if index == torch.cuda.current_device():
+        _launch_on(index, dev, entry, _lib.load().qssm_scan_forward_call)
+    else:
+        with torch.cuda.device(dev):
+            _launch_on(index, dev, entry, _lib.load().qssm_scan_forward_call)
+    return y, h, ckpt, entry.ckpt_stride
+
+
+def _launch_on(index: int, dev: torch.device, entry: _Launch, fn) -> None:
+    """Fill in stream, buffers and epoch of a ready argument block and make the call (device `index` is current)."""
+    stream = _raw_stream(index)
+    buf, epoch, capturing = _launch_buffers(dev, index, stream, entry.need_c, entry.need_w)
+    k = entry.call
+    k.control, k.control_size, k.workspace, k.workspace_bytes = buf.ctl_ptr, buf.ctl_size, buf.ws_ptr, buf.ws_size
+    k.epoch = epoch
+    k.stream = stream
+    rc = fn(entry.call_ref)
+    if rc != 0:
+        _lib.check(rc)
+    _after_launch(buf, stream, capturing)
 
 
 def scan_backward(
@@ -303,8 +473,9 @@ def scan_backward(
     B, L, D = x.shape
     in_dtype = x.dtype
     grads = [torch.empty((B, L, D), dtype=in_dtype, device=dev) if n else None for n in need]
-    for name, t in (("h_init", h_init), ("dh_final", dh_final), ("dh_init", dh_init)):
-        _check_state(t, B, D, dev, name)
+    if h_init is not None or dh_final is not None or dh_init is not None:
+        for name, t in (("h_init", h_init), ("dh_final", dh_final), ("dh_init", dh_init)):
+            _check_state(t, B, D, dev, name)
     if B == 0 or L == 0 or D == 0:
         if dh_init is not None:  # the state passed through untouched
             dh_init.copy_(dh_final) if dh_final is not None else dh_init.zero_()
@@ -317,25 +488,36 @@ def scan_backward(
         h = _unit_inner(h if h.dtype == torch.float32 else h.float())
     else:
         ckpt = ckpt.contiguous()
-    align = _align_elems([x, a, b, c, dy, h, *grads], D)
-    plan = make_plan(B, L, D, in_dtype, dy.dtype, _lib.QSSM_BACKWARD, align, ckpt_stride if h is None else 0, tune)
-    if ckpt is not None and tuple(ckpt.shape) != (B, plan.n_ckpt, D):
-        raise ValueError(f"ckpt has shape {tuple(ckpt.shape)}, expected {(B, plan.n_ckpt, D)}")
+    tensors = (x, a, b, c, dy, h, *grads)
+    strides = tuple(_NO_STRIDE if t is None else t.stride() for t in tensors)
+    ptrs = [None if t is None else t.data_ptr() for t in tensors]
+    align = _align_elems(tensors, D)
+    stride_arg = ckpt_stride if h is None else 0
+    out_dtype = dy.dtype
 
-    with torch.cuda.device(dev):
-        stream = torch.cuda.current_stream(dev).cuda_stream
-        ctl, ws, epoch = _launch_buffers(dev, stream, plan)
-        _lib.check(
-            _lib.load().qssm_scan_backward_carry(
-                ctypes.byref(plan),
-                _ptr(x), _strides(x), _ptr(a), _strides(a), _ptr(b), _strides(b), _ptr(c), _strides(c),
-                _ptr(dy), _strides(dy), _ptr(h), _strides(h), _ptr(ckpt),
-                _ptr(h_init), _ptr(dh_final), _ptr(dh_init),
-                _ptr(grads[0]), _strides(grads[0]), _ptr(grads[1]), _strides(grads[1]),
-                _ptr(grads[2]), _strides(grads[2]), _ptr(grads[3]), _strides(grads[3]),
-                ctl.data_ptr(), ctl.numel(), ws.data_ptr(), ws.numel(), epoch, stream,
-            )
-        )
+    def make() -> _Launch:
+        return _Launch(make_plan(B, L, D, in_dtype, out_dtype, _lib.QSSM_BACKWARD, align, stride_arg, tune), BackwardCall())
+
+    entry = _launch_entry((1, B, L, D, in_dtype, out_dtype, align, stride_arg, tune), make)
+    if ckpt is not None and tuple(ckpt.shape) != (B, entry.n_ckpt, D):
+        raise ValueError(f"ckpt has shape {tuple(ckpt.shape)}, expected {(B, entry.n_ckpt, D)}")
+
+    k = entry.call
+    if entry.strides != strides:
+        (k.sx, k.sa, k.sb, k.sc, k.sdy, k.sh, k.sdx, k.sda, k.sdb, k.sdc) = (Strides(s[0], s[1]) for s in strides)
+        entry.strides = strides
+    k.x, k.a, k.b, k.c, k.dy, k.h, k.dx, k.da, k.db, k.dc = ptrs
+    k.ckpt = None if ckpt is None else ckpt.data_ptr()
+    k.h_init = None if h_init is None else h_init.data_ptr()
+    k.dh_final = None if dh_final is None else dh_final.data_ptr()
+    k.dh_init = None if dh_init is None else dh_init.data_ptr()
+
+    index = dev.index
+    if index == torch.cuda.current_device():
+        _launch_on(index, dev, entry, _lib.load().qssm_scan_backward_call)
+    else:
+        with torch.cuda.device(dev):
+            _launch_on(index, dev, entry, _lib.load().qssm_scan_backward_call)
     return tuple(grads)
 
 

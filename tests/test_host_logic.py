@@ -68,7 +68,7 @@ def test_plan_rejects_bad_arguments(hip_lib):
         hip_scan.make_plan(1, 64, 4, torch.float32, torch.float32, 0, 4, ckpt_stride=48)
     assert "power of two" in str(err.value)
     plan = _lib.Plan()
-    rc = hip_lib.qssm_plan_scan(1, 4, 4, 7, 0, 0, 4, 0, 0, ctypes.byref(plan))
+    rc = hip_lib.qssm_plan_scan(1, 4, 4, 7, 0, 0, 4, 0, ctypes.byref(plan))
     assert rc == _lib.QSSM_EINVAL and b"dtype" in hip_lib.qssm_error_string()
     # fp32 operands with 16-bit y is not a built pair: the host casts instead
     assert hip_scan.kernel_dtypes([torch.float32] * 4, torch.float16) == (torch.float32, torch.float32)

@@ -381,7 +381,7 @@ def test_dirty_control_block_is_reported_and_zero_fill_recovers(gpu):
     none = _lib.Strides(0, 0)
 
     def launch(epoch):
-        y = torch.full(shape, float("nan"), dtype=torch.float16, device=gpu)
+        y = torch.zeros(shape, dtype=torch.float16, device=gpu)
         _lib.check(lib.qssm_scan_forward(
             ctypes.byref(plan), ops[0].data_ptr(), st(ops[0]), ops[1].data_ptr(), st(ops[1]), ops[2].data_ptr(), st(ops[2]),
             ops[3].data_ptr(), st(ops[3]), y.data_ptr(), st(y), None, none, None,
@@ -391,12 +391,84 @@ def test_dirty_control_block_is_reported_and_zero_fill_recovers(gpu):
         return y, status.value
 
     y, status = launch(1)
-    assert status == 2 and torch.isnan(y).all()           # nothing was written
+    assert status == 2 and torch.isnan(y).all()           # every tile of the output was poisoned, nothing else ran
     _lib.check(lib.qssm_zero_fill(control.data_ptr(), control.numel(), stream))
     y, status = launch(2)
     assert status == 0
     _, y64 = oracle.forward_f64(x, a, b, c)
     assert_close("y", y.cpu(), y64, TOL[torch.float16])
+
+
+def test_failed_launch_is_reported_through_scan_and_the_stream_recovers(gpu):
+    # The same dirty control block, this time under the public API: the launch poisons its outputs, the status
+    # check behind it (period 1 here) brings the word to the host, the next scan() on the stream raises
+    # ScanLaunchError after resetting the buffers, and the one after that is correct again.  Every kernel exits
+    # normally throughout.
+    shape = (2, 700, 256)
+    x, a, b, c, dy = make_inputs(shape, dtype=torch.bfloat16, seed=72)
+    ops = [t.to(gpu) for t in (x, a, b, c)]
+    old = hip_scan.set_status_check_period(1)
+    try:
+        y = scan(*ops)                                     # the buffers of this stream exist and are large enough
+        torch.cuda.synchronize()
+        stream = torch.cuda.current_stream(gpu).cuda_stream
+        buf = hip_scan._buffers[(gpu.index, stream, False)]
+        buf.control.view(torch.int32)[16:] = 0x7fff0000    # every ticket slot; the status word stays zero
+        y = scan(*ops)
+        torch.cuda.synchronize()
+        assert torch.isnan(y).all()
+        with pytest.raises(hip_scan.ScanLaunchError) as err:
+            scan(*ops)
+        assert err.value.status == 2
+        got = run_scan_with_grads(scan, x, a, b, c, dy, gpu)
+        assert hip_scan.workspace_status() == 0
+        _check_all(got, oracle_all(x, a, b, c, dy), TOL[torch.bfloat16])
+    finally:
+        hip_scan.set_status_check_period(old)
+
+
+def test_buffers_of_a_recorded_graph_outlive_a_larger_shape(gpu):
+    # A graph recorded for a small shape holds the addresses of its control block and workspace.  A larger shape on
+    # the same stream needs larger buffers: the old pair must stay alive and untouched (it is retired, not freed),
+    # and the old graph must still replay correctly afterwards.
+    small, large = (1, 600, 256), (4, 4096, 1024)
+    side = torch.cuda.Stream()
+    xs = [t.to(gpu).contiguous() for t in make_inputs(small, dtype=torch.bfloat16, seed=81)]
+    xl = [t.to(gpu).contiguous() for t in make_inputs(large, dtype=torch.bfloat16, seed=82)]
+
+    def run(ops):
+        y, _, ckpt, stride = hip_scan.scan_forward(*ops[:4], out_dtype=torch.bfloat16)
+        return (y,) + tuple(hip_scan.scan_backward(*ops, ckpt=ckpt, ckpt_stride=stride))
+
+    with torch.cuda.stream(side):
+        with hip_scan.device_counted_launches():
+            run(xs)
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            outs = run(xs)
+        key = (gpu.index, side.cuda_stream, True)
+        before = hip_scan._buffers[key]
+        old_ptrs = (before.ctl_ptr, before.ws_ptr)
+        assert before.captured
+        retired = len(hip_scan._retired)
+        with hip_scan.device_counted_launches():
+            big = run(xl)                                   # needs a larger workspace than the recorded pair
+        side.synchronize()
+        after = hip_scan._buffers[key]
+        assert after.ws_ptr != old_ptrs[1] and len(hip_scan._retired) == retired + 2
+        assert {t.data_ptr() for t in hip_scan._retired[-2:]} == set(old_ptrs)
+        fresh = make_inputs(small, dtype=torch.bfloat16, seed=83)
+        for dst, src in zip(xs, fresh):
+            dst.copy_(src.to(gpu))
+        for _ in range(2):
+            graph.replay()
+            side.synchronize()
+            got = dict(zip(("y", "dx", "da", "db", "dc"), (t.cpu() for t in outs)))
+            _check_all(got, oracle_all(*fresh), TOL[torch.bfloat16])
+        assert hip_scan.workspace_status() == 0
+        ref = oracle_all(*make_inputs(large, dtype=torch.bfloat16, seed=82))
+        _check_all(dict(zip(("y", "dx", "da", "db", "dc"), (t.cpu() for t in big))), ref, TOL[torch.bfloat16])
 
 
 def test_captured_launches_replay_with_new_inputs(gpu):
@@ -413,10 +485,13 @@ def test_captured_launches_replay_with_new_inputs(gpu):
         y, _, ckpt, stride = hip_scan.scan_forward(*static[:4], out_dtype=torch.bfloat16, tune=tune, bwd_tune=tune)
         return (y,) + tuple(hip_scan.scan_backward(*static, ckpt=ckpt, ckpt_stride=stride, tune=tune))
 
+    import warnings
     with torch.cuda.stream(side):
-        with pytest.raises(RuntimeError):   # recording the very first launch would have to allocate
-            with torch.cuda.graph(torch.cuda.CUDAGraph(), stream=side):
-                run()
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")     # torch warns that the graph of the refused recording is empty
+            with pytest.raises(RuntimeError):   # recording the very first launch would have to allocate
+                with torch.cuda.graph(torch.cuda.CUDAGraph(), stream=side):
+                    run()
         with hip_scan.device_counted_launches():   # warm-up: the buffers of captured launches exist afterwards
             run()
         run()
@@ -424,8 +499,12 @@ def test_captured_launches_replay_with_new_inputs(gpu):
         plan = hip_scan.make_plan(*shape, torch.bfloat16, torch.bfloat16, _lib.QSSM_BACKWARD, 8, 0, tune)
         assert plan.n_seg > 1 and plan.n_super > 1
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=side):
-            outs = run()
+        with warnings.catch_warnings():
+            warnings.simplefilter("error")      # the real recording must not be empty
+            with torch.cuda.graph(graph, stream=side):
+                outs = run()
+        for t in outs:
+            t.fill_(float("nan"))               # whatever the outputs hold later, a replay wrote it
     for k in (1, 2, 0, 1):
         for dst, src in zip(static, sets[k]):
             dst.copy_(src.to(gpu))

@@ -30,7 +30,7 @@ def _forward_both_ways(lib, gpu, shape, dtype, seed):
     code = {torch.float32: _lib.QSSM_F32, torch.float16: _lib.QSSM_F16, torch.bfloat16: _lib.QSSM_BF16}[dtype]
     stride = hip_scan.make_plan(B, L, D, dtype, dtype, _lib.QSSM_BACKWARD, 8, 0).seg_len
     plan = Plan()
-    assert lib.qssm_plan_scan(B, L, D, code, code, _lib.QSSM_FORWARD, 8, stride, 0, ctypes.byref(plan)) == 0
+    assert lib.qssm_plan_scan(B, L, D, code, code, _lib.QSSM_FORWARD, 8, stride, ctypes.byref(plan)) == 0
     xd, ad, bd, cd = (t.to(gpu) for t in (x, a, b, c))
     stream = torch.cuda.current_stream(gpu).cuda_stream
     none = Strides(0, 0)
@@ -76,7 +76,7 @@ def test_static_entry_point_refuses_what_does_not_fit(gpu, hip_lib):
     lib = hip_lib
     B, L, D = 64, 8192, 4096     # 8.6 G elements' worth of tiles: far more workspace than the array holds
     plan = Plan()
-    assert lib.qssm_plan_scan(B, L, D, _lib.QSSM_BF16, _lib.QSSM_BF16, _lib.QSSM_FORWARD, 8, 32, 0,
+    assert lib.qssm_plan_scan(B, L, D, _lib.QSSM_BF16, _lib.QSSM_BF16, _lib.QSSM_FORWARD, 8, 32,
                               ctypes.byref(plan)) == 0
     assert plan.workspace_bytes > _lib.QSSM_STATIC_SCRATCH_BYTES
     t = torch.zeros(8, dtype=torch.bfloat16, device=gpu)     # never touched: the call is refused first
