@@ -65,9 +65,21 @@ def event_time_ms(torch, fn, iters, warmup):
     return start.elapsed_time(stop) / iters
 
 
+def kernel_source_hash() -> str:
+    """Hash of the scan kernels' sources: measured traffic is only quoted for the kernels it was measured on."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in ("scan_common.h", "scan_fwd.hip", "scan_bwd.hip"):
+        h.update((ROOT / "quick_ssm_amd" / "csrc" / name).read_bytes())
+    return h.hexdigest()[:16]
+
+
 def cpu_baseline(torch, workload, shape, dtype, out_dtype, a_lo, a_span):
-    """The reference CPU path (torch restatement, oracle/reference_cpu_path.py) on a bounded slice."""
-    from oracle.reference_cpu_path import reference_scan_with_grads
+    """The reference CPU path (torch restatement, oracle/reference_cpu_path.py) on a bounded slice, plus the two legs
+    the path can do in full: the fp32 B=4 L=2048 D=16 configuration forward + backward, and this workload's forward
+    at full shape under no_grad (both bounded by the clock: rows stop being added after 8 s)."""
+    from oracle.reference_cpu_path import reference_scan, reference_scan_with_grads
 
     B, L, D = shape
     # One batch row with every column of the workload.  The reference's backward through its in-place slice writes
@@ -85,7 +97,7 @@ def cpu_baseline(torch, workload, shape, dtype, out_dtype, a_lo, a_span):
     n = sB * sL * sD
     es, os_ = ops[0].element_size(), ops[4].element_size()
     nbytes = n * (8 * es + 2 * os_)
-    return {
+    out = {
         "value": nbytes / dt / 1e9,
         "unit": "GB/s",
         "cores": torch.get_num_threads(),
@@ -95,6 +107,29 @@ def cpu_baseline(torch, workload, shape, dtype, out_dtype, a_lo, a_span):
         "melem_per_s": n / dt / 1e6,
         "seconds": dt,
     }
+    # the configuration the reference's CPU path runs in full: fp32 B=4 L=2048 D=16, forward + backward
+    c0 = WORKLOADS["c0"]
+    ops0, _ = make_operands(torch, c0[:3], torch.float32, torch.float32, c0[5], c0[6], "cpu")
+    t0 = time.perf_counter()
+    reference_scan_with_grads(*ops0, out_dtype=torch.float32)
+    dt0 = time.perf_counter() - t0
+    n0 = c0[0] * c0[1] * c0[2]
+    out["c0_full"] = {"seconds": dt0, "melem_per_s": n0 / dt0 / 1e6, "gbs": n0 * 14 * 4 / dt0 / 1e9,
+                      "sample": "fp32 B=4 L=2048 D=16 fwd+bwd, whole configuration"}
+    # this workload's forward at its full shape under no_grad, batch row by batch row until the clock says stop
+    with torch.no_grad():
+        done, dtf = 0, 0.0
+        ops1, _ = make_operands(torch, (1, L, D), dtype, out_dtype, a_lo, a_span, "cpu")
+        while done < B and dtf < 8.0:
+            t0 = time.perf_counter()
+            reference_scan(*ops1[:4], out_dtype=out_dtype)
+            dtf += time.perf_counter() - t0
+            done += 1
+    nf = done * L * D
+    out["forward_full_shape"] = {"seconds": dtf, "rows_done": done, "rows": B, "melem_per_s": nf / dtf / 1e6,
+                                 "gbs": nf * (4 * es + os_) / dtf / 1e9,
+                                 "sample": f"forward only, no_grad, L={L} D={D}, {done} of {B} batch rows"}
+    return out
 
 
 def main() -> int:
@@ -208,11 +243,17 @@ def main() -> int:
     plan_b = hip_scan.make_plan(B, L, D, dtype, out_dtype, _lib.QSSM_BACKWARD, align, stride)
     plan_f = hip_scan.make_plan(B, L, D, dtype, out_dtype, _lib.QSSM_FORWARD, align, stride)
 
-    traffic = None
+    # HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this command: only
+    # quoted while the kernels are the ones it was measured on
+    traffic, traffic_note = None, "not measured for this workload"
     traffic_file = ROOT / "profiles" / f"scan_bwd_{args.workload}_traffic.json"
     if traffic_file.exists():
         try:
-            traffic = json.loads(traffic_file.read_text()).get("traffic_bytes_per_launch")
+            rec = json.loads(traffic_file.read_text())
+            if rec.get("kernel_source_hash") == kernel_source_hash():
+                traffic, traffic_note = rec.get("traffic_bytes_per_launch"), rec.get("source", "")
+            else:
+                traffic_note = "kernel sources changed since profiles/ was measured"
         except (ValueError, OSError):
             traffic = None
 
@@ -220,7 +261,7 @@ def main() -> int:
     fwd_gbs = fwd_bytes / (fwd_ms * 1e-3) / 1e9
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
     out = {
-        "metric": "scan fwd+bwd HBM GB/s (% of peak) + Melem/s, bf16 B=8 L=4096 D=2048",
+        "metric": f"scan fwd+bwd HBM GB/s (% of peak) + Melem/s, {desc}",
         "value": value,
         "unit": "GB/s",
         "n_gpus": 1,
@@ -248,6 +289,7 @@ def main() -> int:
             "unit": "GB/s",
             "frac": bwd_gbs / HBM_PEAK_GBS,
             "traffic": traffic,
+            "traffic_note": traffic_note,
             "algorithmic_bytes_per_launch": bwd_bytes,
             "avg_launch_ms": bwd_ms,
         },

@@ -1,7 +1,7 @@
 """Times the SSM layer's HIP passes around the scan, and the layer step they sit in, on one GPU.
 
-    python -m quick_ssm_amd.layer_bench [--batch 16] [--length 2048] [--hidden 1024] [--mult 4.0]
-                                        [--param-dtype float32] [--compute-dtype float16] [--steps 20] [--warmup 5]
+    python layer_bench.py [--batch 16] [--length 2048] [--hidden 1024] [--mult 4.0]
+                          [--param-dtype float32] [--compute-dtype float16] [--steps 20] [--warmup 5]
 
 Defaults are the layer configuration of the reference's example scripts (quick_ssm/example_layer.py,
 copy_train.py:26: state = 4 x hidden, fp32 parameters, fp16 scan operands).  Each pass is timed alone
@@ -22,6 +22,11 @@ from __future__ import annotations
 import argparse
 import json
 import sys
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0
 
@@ -53,7 +58,7 @@ def main() -> int:
 
     import torch
 
-    from . import _lib, gates, hip_scan, layers, norm
+    from quick_ssm_amd import _lib, gates, hip_scan, layers, norm
 
     if not torch.cuda.is_available():
         print("layer_bench needs a GPU", file=sys.stderr)

@@ -96,7 +96,8 @@ static int check_plan(const qssm_plan* pl, int direction) {
   if (pl == nullptr) return fail(QSSM_EINVAL, "plan is NULL");
   if (pl->direction != direction) return fail(QSSM_EINVAL, "plan was made for the other direction");
   if (pl->B < 0 || pl->L < 0 || pl->D < 0) return fail(QSSM_EINVAL, "negative dimension");
-  if (pl->vec != 1 && pl->vec != 2 && pl->vec != 4) return fail(QSSM_EINVAL, "plan.vec must be 1, 2 or 4");
+  if (pl->vec != 1 && pl->vec != 2 && pl->vec != 4 && !(pl->vec == 8 && direction == QSSM_FORWARD && dtype_size(pl->in_dtype) == 2))
+    return fail(QSSM_EINVAL, "plan.vec must be 1, 2 or 4 (8 for a forward over 16-bit storage)");
   if (pl->steps != 4 && pl->steps != 8) return fail(QSSM_EINVAL, "plan.steps must be 4 or 8");
   if (!threads_ok(pl->threads)) return fail(QSSM_EINVAL, "plan.threads must be 256, 512 or 1024");
   if (pl->g_log2 < 0 || (1 << pl->g_log2) > pl->threads) return fail(QSSM_EINVAL, "plan.g_log2 out of range");
@@ -216,6 +217,15 @@ int qssm_plan_scan_tuned(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int3
   if (es == 4 && direction == QSSM_BACKWARD) vec = 2;
   const int tune_vec = (tune >> 16) & 0xff;
   if (tune_vec == 1 || tune_vec == 2) vec = tune_vec < vec ? tune_vec : vec;
+  // The forward over 16-bit storage takes 16 bytes per lane (8 columns) when the launch is large enough to fill the
+  // GPU with such tiles: half the wavefronts per tile for the same bytes, and every load, store and LDS access
+  // twice as wide (bf16 B=8 L=4096 D=2048: 124 us against 130 with 8 bytes per lane).  Its register footprint
+  // (a, b, x of 8 steps: 96 registers) does not leave room for the backward's rebuilt states, so the backward
+  // stays at 8 bytes per lane (16 bytes at 4 steps per lane measured 240 us against 220).
+  const bool wide_ok = direction == QSSM_FORWARD && es == 2 && align_elems % 8 == 0 && D % 8 == 0;
+  const bool wide_auto = direction == QSSM_FORWARD && tune_vec == 0 && os == 2 && D >= 256 &&
+                         (int64_t)B * ((D + 255) / 256) * ((L + 63) / 64) >= 2 * kCUs;
+  if (wide_ok && (tune_vec == 8 || wide_auto)) vec = 8;
   while (vec > 1 && (align_elems % vec != 0 || (D > 0 && D % vec != 0))) vec >>= 1;
   plan->vec = vec;
 
@@ -235,6 +245,7 @@ int qssm_plan_scan_tuned(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int3
   // The forward for 16-bit storage keeps c in LDS when rows can be fetched 16 bytes at a time, which
   // leaves room for two 512-lane workgroups per compute unit: tiles twice as long, half the hand-overs.
   if (direction == QSSM_FORWARD && es == 2 && vec == 4 && steps == 8 && align_elems % 8 == 0) threads = 512;
+  if (vec == 8) threads = 256;
   const int tune_g = (tune & 0xff) - 1, tune_t = (tune >> 24) & 0xf;
   const bool fixed_g = tune_g >= 0 && tune_g <= 10, fixed_t = tune_t >= 1 && tune_t <= 3;
   if (fixed_g) g = 1 << tune_g;
@@ -283,7 +294,7 @@ int qssm_plan_scan_tuned(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int3
     if ((ckpt_stride & (ckpt_stride - 1)) != 0 || ckpt_stride < 4)
       return fail(QSSM_EINVAL, "ckpt_stride=%d must be a power of two >= 4", ckpt_stride);
     if (direction == QSSM_FORWARD && ckpt_stride % steps != 0) steps = 4;
-    while (steps * (threads / g) < ckpt_stride && threads < kMaxThreads && vec > 1) threads <<= 1;
+    while (steps * (threads / g) < ckpt_stride && threads < kMaxThreads && vec > 1 && vec < 8) threads <<= 1;
     while (steps * (threads / g) < ckpt_stride && g > 1) g >>= 1;
     if ((steps * (threads / g)) % ckpt_stride != 0)
       return fail(QSSM_EINVAL, "ckpt_stride=%d does not fit any tile length", ckpt_stride);
@@ -321,6 +332,13 @@ int qssm_plan_scan_tuned(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int3
   } else {
     while (cluster < 8 && (plan->n_seg + cluster - 1) / cluster > 64) cluster <<= 1;
     if (cluster < 2 && plan->n_seg > 8) cluster = 2;
+    // A chain of single tiles exchanges the fewest words (no maps at all, 1.9 % less traffic on the forward than
+    // clusters of two), and hands a state on in about 2.1 us.  Where a chain of that many hand-overs still ends
+    // well inside the time the launch needs to stream its operands (taken at 5.6 TB/s), it is the better trade
+    // (bf16 B=16 L=4096 D=2048 forward: 233 us against 237); where it does not (the same at B=8: 64 hand-overs in
+    // 116 us), the chain would set the pace and clusters stay.
+    const double stream_us = (double)B * L * D * (direction == QSSM_FORWARD ? 4 * es + os : 8 * es + os) / 5.6e6;
+    if (cluster > 1 && plan->n_seg * 2.1 <= 0.6 * stream_us) cluster = 1;
   }
   auto lds_for = [&](int r) -> size_t {
     return direction == QSSM_FORWARD ? fwd_lds_bytes(threads, vec, plan->strip_cols, r)
@@ -447,11 +465,12 @@ static int forward_launch(const qssm_plan* plan, const void* x, qssm_strides sx,
   // c can live in LDS instead of registers when a row of the strip is one wavefront of 8-byte lanes
   // and c's rows can be fetched 16 bytes at a time.
   size_t lds = (size_t)plan->lds_bytes;
-  bool c_in_lds = y != nullptr && c != nullptr && es == 2 && v == 4 && (plan->g_log2 == 6 || plan->g_log2 == 5) && plan->steps == 8 &&
-                  (plan->threads == 256 || plan->threads == 512) && ((uintptr_t)c) % 16 == 0 &&
-                  (sc.b * es) % 16 == 0 && (sc.l * es) % 16 == 0 &&
-                  lds + fwd_c_lds_bytes(plan->threads, plan->steps) <= (size_t)kMaxLdsBytes;
-  if (c_in_lds) lds += fwd_c_lds_bytes(plan->threads, plan->steps);
+  const bool narrow_rows = v == 4 && (plan->g_log2 == 6 || plan->g_log2 == 5) && (plan->threads == 256 || plan->threads == 512);
+  const bool wide_rows = v == 8 && (plan->threads == 256 || plan->threads == 512);   // every lane fetches its own 16 bytes
+  bool c_in_lds = y != nullptr && c != nullptr && es == 2 && ((narrow_rows && plan->steps == 8) || wide_rows) &&
+                  ((uintptr_t)c) % 16 == 0 && (sc.b * es) % 16 == 0 && (sc.l * es) % 16 == 0 &&
+                  lds + fwd_c_lds_bytes(plan->threads, plan->steps, v * es) <= (size_t)kMaxLdsBytes;
+  if (c_in_lds) lds += fwd_c_lds_bytes(plan->threads, plan->steps, v * es);
   if (!fn(args, plan->vec, plan->steps, plan->threads, c_in_lds, grid, lds, (hipStream_t)stream))
     return fail(QSSM_EINVAL, "no forward kernel for vec=%d steps=%d threads=%d", plan->vec, plan->steps, plan->threads);
   if (epoch == 0 && plan->n_seg > 1)

@@ -54,7 +54,12 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   auto lds_row = [&](int i) { return (i >> 1) * 1024 + (i & 1) * (G * 8); };
 
   const int tid = threadIdx.x;
-  const int chain = blockIdx.x % g.n_chains;
+  // Workgroups go to the eight XCDs in turn, so workgroup i runs on XCD i mod 8.  Chains are dealt out so that each
+  // XCD gets a run of adjacent chains (the strips of one batch row, when there are eight of each) rather than
+  // every eighth one: its workgroups then stream whole rows of few batch rows instead of one 512-byte column of
+  // all of them, which its L2 and address translation reward.  All tiles of a chain still run on one XCD.
+  int chain = blockIdx.x % g.n_chains;
+  if ((g.n_chains & 7) == 0) chain = (chain & 7) * (g.n_chains >> 3) + (chain >> 3);
 
   // ---- claim a tile of this chain, last tile in time first -----------------------------------
   int seg = 0;

@@ -74,7 +74,7 @@ typedef _Float16 f16_t;
 typedef __bf16 bf16_t;
 
 template <typename T, int V>
-struct alignas(sizeof(T) * V) Pack {
+struct alignas(sizeof(T) * V > 16 ? 16 : sizeof(T) * V) Pack {
   T v[V];
 };
 
@@ -155,6 +155,13 @@ __device__ __forceinline__ float elem(const Words<T, V>& p, int v) {
 // Operands and results are touched exactly once, so they are marked non-temporal (streaming).
 template <typename T, int V>
 __device__ __forceinline__ Words<T, V> load_stream(const char* base, uint32_t byte_off) {
+  if constexpr (sizeof(T) * V == 32) {   // two 16-byte halves
+    const Words<T, V / 2> lo = load_stream<T, V / 2>(base, byte_off), hi = load_stream<T, V / 2>(base, byte_off + 16u);
+    Words<T, V> out;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) { out.w[k] = lo.w[k]; out.w[4 + k] = hi.w[k]; }
+    return out;
+  } else {
   typedef typename RawOf<sizeof(T) * V>::type raw_t;
   const raw_t r = __builtin_nontemporal_load(reinterpret_cast<const raw_t*>(base + byte_off));
   Words<T, V> out;
@@ -165,10 +172,15 @@ __device__ __forceinline__ Words<T, V> load_stream(const char* base, uint32_t by
     for (int k = 0; k < Words<T, V>::N; ++k) out.w[k] = r[k];
   }
   return out;
+  }
 }
 
 template <typename T, int V>
 __device__ __forceinline__ void store_stream(char* base, uint32_t byte_off, const float* f) {
+  if constexpr (sizeof(T) * V == 32) {   // two 16-byte halves
+    store_stream<T, V / 2>(base, byte_off, f);
+    store_stream<T, V / 2>(base, byte_off + 16u, f + V / 2);
+  } else {
   typedef typename RawOf<sizeof(T) * V>::type raw_t;
   Words<T, V> p;
   ElemBits<T>::template set<V>(p, f);
@@ -180,6 +192,7 @@ __device__ __forceinline__ void store_stream(char* base, uint32_t byte_off, cons
     for (int k = 0; k < Words<T, V>::N; ++k) r[k] = p.w[k];
   }
   __builtin_nontemporal_store(r, reinterpret_cast<raw_t*>(base + byte_off));
+  }
 }
 
 // All VEC elements equal to 1 (`one`) or 0.
@@ -195,15 +208,31 @@ __device__ __forceinline__ Words<T, V> fill_words(bool one) {
 
 template <typename T, int V>
 __device__ __forceinline__ Pack<T, V> load_pack(const T* p) {
-  typedef typename RawOf<sizeof(T) * V>::type raw_t;
-  raw_t r = *reinterpret_cast<const raw_t*>(p);
-  return __builtin_bit_cast(Pack<T, V>, r);
+  if constexpr (sizeof(T) * V == 32) {   // two 16-byte halves
+    const Pack<T, V / 2> lo = load_pack<T, V / 2>(p), hi = load_pack<T, V / 2>(p + V / 2);
+    Pack<T, V> out;
+#pragma unroll
+    for (int k = 0; k < V / 2; ++k) { out.v[k] = lo.v[k]; out.v[V / 2 + k] = hi.v[k]; }
+    return out;
+  } else {
+    typedef typename RawOf<sizeof(T) * V>::type raw_t;
+    raw_t r = *reinterpret_cast<const raw_t*>(p);
+    return __builtin_bit_cast(Pack<T, V>, r);
+  }
 }
 
 template <typename T, int V>
 __device__ __forceinline__ void store_pack(T* p, const Pack<T, V>& v) {
-  typedef typename RawOf<sizeof(T) * V>::type raw_t;
-  *reinterpret_cast<raw_t*>(p) = __builtin_bit_cast(raw_t, v);
+  if constexpr (sizeof(T) * V == 32) {   // two 16-byte halves
+    Pack<T, V / 2> lo, hi;
+#pragma unroll
+    for (int k = 0; k < V / 2; ++k) { lo.v[k] = v.v[k]; hi.v[k] = v.v[V / 2 + k]; }
+    store_pack<T, V / 2>(p, lo);
+    store_pack<T, V / 2>(p + V / 2, hi);
+  } else {
+    typedef typename RawOf<sizeof(T) * V>::type raw_t;
+    *reinterpret_cast<raw_t*>(p) = __builtin_bit_cast(raw_t, v);
+  }
 }
 
 // VEC adjacent floats in LDS as one access (a lane's VEC columns sit next to each other, so a
@@ -414,8 +443,8 @@ inline size_t bwd_lds_bytes(int nth, int vec, int cols, int cluster) {
 // Return false if (vec, steps, threads) is not an instantiated combination.
 typedef bool (*fwd_launch_fn)(const FwdArgs&, int vec, int steps, int threads, bool c_in_lds, dim3 grid, size_t lds,
                               hipStream_t stream);
-// Extra dynamic LDS of the forward kernel that keeps c in LDS: 8 bytes per lane and step.
-inline size_t fwd_c_lds_bytes(int nth, int steps) { return (size_t)nth * steps * 8; }
+// Extra dynamic LDS of the forward kernel that keeps c in LDS: 8 or 16 bytes per lane and step.
+inline size_t fwd_c_lds_bytes(int nth, int steps, int lane_bytes) { return (size_t)nth * steps * lane_bytes; }
 typedef bool (*bwd_launch_fn)(const BwdArgs&, int vec, int steps, int threads, bool cg_in_lds, dim3 grid, size_t lds,
                               hipStream_t stream);
 // Extra dynamic LDS of the backward kernel that keeps c and dy in LDS.

@@ -21,7 +21,11 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // 8 bytes per lane, so that one wavefront-wide 16-byte-per-lane load covers whole rows of the strip.
 template <typename Tin, typename Tout, int VEC, int T, int NTH, bool CLDS>
 __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
-  static_assert(!CLDS || (sizeof(Tin) * VEC == 8 && T % 2 == 0), "LDS-resident c: 8 bytes per lane, even step count");
+  static_assert(!CLDS || ((sizeof(Tin) * VEC == 8 || sizeof(Tin) * VEC == 16) && T % 2 == 0),
+                "LDS-resident c: 8 or 16 bytes per lane, even step count");
+  // 16 bytes per lane: the load that deposits c in LDS gives every lane exactly its own columns of one step.
+  constexpr bool WIDE = sizeof(Tin) * VEC == 16;
+  constexpr int CROW = WIDE ? 1024 : 512;   // bytes of c one wavefront holds per step
   extern __shared__ __align__(16) float lds[];
   const Geometry& g = p.g;
   const int G = 1 << g.g_log2;
@@ -36,14 +40,19 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   float* sPX = sPA + (R - 1) * cols;
   float* sH = sPX + (R - 1) * cols;      // [cols] state entering the tile
   int* sSeg = reinterpret_cast<int*>(sH + cols);
-  char* sC = reinterpret_cast<char*>(sSeg) + 16;  // CLDS: [NTH / 64 waves][T rows][512 bytes] of c
+  char* sC = reinterpret_cast<char*>(sSeg) + 16;  // CLDS: [NTH / 64 waves][T rows][CROW bytes] of c
 
   const int tid = threadIdx.x;
-  const int chain = blockIdx.x % g.n_chains;
+  // Workgroups go to the eight XCDs in turn, so workgroup i runs on XCD i mod 8.  Chains are dealt out so that each
+  // XCD gets a run of adjacent chains (the strips of one batch row, when there are eight of each) rather than
+  // every eighth one: its workgroups then stream whole rows of few batch rows instead of one 512-byte column of
+  // all of them, which its L2 and address translation reward.  All tiles of a chain still run on one XCD.
+  int chain = blockIdx.x % g.n_chains;
+  if ((g.n_chains & 7) == 0) chain = (chain & 7) * (g.n_chains >> 3) + (chain >> 3);
   // Where step i of this lane sits in its wavefront's block of sC: the loads that fill it deposit 1024 bytes
   // per instruction in lane order, i.e. per pair of steps [group in wavefront][step parity][G * 8 bytes].
-  const int lds_lane = ((tid & 63) >> g.g_log2) * (G * 16) + (tid & (G - 1)) * 8;
-  auto lds_row = [&](int i) { return (i >> 1) * 1024 + (i & 1) * (G * 8); };
+  const int lds_lane = WIDE ? (tid & 63) * 16 : ((tid & 63) >> g.g_log2) * (G * 16) + (tid & (G - 1)) * 8;
+  auto lds_row = [&](int i) { return WIDE ? i * 1024 : (i >> 1) * 1024 + (i & 1) * (G * 8); };
 
   // ---- claim a tile of this chain, in time order -------------------------------------------
   int seg = 0;
@@ -127,7 +136,12 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
       rb[i] = load_stream<Tin, VEC>(bb, bo + i * bs);
       rx[i] = load_stream<Tin, VEC>(xb, xo + i * xs);
     }
-    if (CLDS) {
+    if (CLDS && WIDE) {
+      char* dst = sC + (tid >> 6) * (T * CROW);
+#pragma unroll
+      for (int i = 0; i < T; ++i)
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(cb + co + i * cs), (lds_ptr_t)(dst + i * 1024), 16, 0, 2);
+    } else if (CLDS) {
       // 16 bytes per lane: the first half of a lane group's lanes fetches one row of the strip, the second half
       // the next one (64 lanes per row: a wavefront covers two rows of one group; 32: two rows of two groups)
       const int wl = tid & 63;
@@ -162,7 +176,7 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
     if (CLDS) {
       // Ragged tile: c goes through a register one step at a time (rare, and kept rolled up so that
       // it does not bring the sixteen registers back).
-      char* dst = sC + (tid >> 6) * (T * 512) + lds_lane;
+      char* dst = sC + (tid >> 6) * (T * CROW) + lds_lane;
 #pragma unroll 1
       for (int i = 0; i < T; ++i) {
         Words<Tin, VEC> cw = fill_words<Tin, VEC>(false);
@@ -342,7 +356,7 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   for (int i = 0; i < T; ++i) {
     float yv[VEC];
     Words<Tin, VEC> cw;
-    if (CLDS) cw = *reinterpret_cast<const Words<Tin, VEC>*>(sC + (tid >> 6) * (T * 512) + lds_row(i) + lds_lane);
+    if (CLDS) cw = *reinterpret_cast<const Words<Tin, VEC>*>(sC + (tid >> 6) * (T * CROW) + lds_row(i) + lds_lane);
     else cw = rc[i];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
@@ -377,6 +391,12 @@ static bool launch_fwd(const FwdArgs& args, int vec, int steps, int threads, boo
   if constexpr (sizeof(Tin) == 2) {
     QSSM_FWD_CASE(4, 8, 256, true)
     QSSM_FWD_CASE(4, 8, 512, true)
+    QSSM_FWD_CASE(8, 8, 256, true)
+    QSSM_FWD_CASE(8, 8, 256, false)
+    QSSM_FWD_CASE(8, 4, 256, true)
+    QSSM_FWD_CASE(8, 4, 256, false)
+    QSSM_FWD_CASE(8, 4, 512, true)
+    QSSM_FWD_CASE(8, 4, 512, false)
   }
   QSSM_FWD_CASE(1, 4, 256, false)
   QSSM_FWD_CASE(1, 8, 256, false)

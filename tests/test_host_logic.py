@@ -200,6 +200,13 @@ def test_tile_index_arithmetic_stays_in_bounds(hip_lib, shape, dtype):
             assert lo >= 0 and hi == B * L * D - 1          # every element is covered, nothing beyond
             assert hi_ckpt < plan.ckpt_elems
             assert hi_word <= plan.workspace_bytes
+    if dtype != torch.float32 and D % 8 == 0:
+        # the forward with 8 columns (16 bytes) per lane, forced onto these small shapes
+        for tune in (8 << 16, 3 | (8 << 16) | (3 << 28), 6 | (8 << 16) | (2 << 28)):
+            plan = hip_scan.make_plan(B, L, D, dtype, dtype, _lib.QSSM_FORWARD, 8, 32, tune)
+            assert plan.vec == 8 and plan.threads == 256
+            lo, hi, hi_ckpt, hi_word = _tile_accesses(plan, B, L, D)
+            assert lo >= 0 and hi == B * L * D - 1 and hi_ckpt < plan.ckpt_elems and hi_word <= plan.workspace_bytes
 
 
 def test_plan_invariants_over_random_shapes(hip_lib):
@@ -220,7 +227,8 @@ def test_plan_invariants_over_random_shapes(hip_lib):
         fwd = hip_scan.make_plan(B, L, D, dt, odt, _lib.QSSM_FORWARD, align, bwd.seg_len)
         for p in (bwd, fwd):
             what = (B, L, D, dt, odt, align, p.describe())
-            assert p.vec in (1, 2, 4) and D % p.vec == 0 and align % p.vec == 0, what
+            wide = p is fwd and dt != torch.float32 and odt == dt     # 16 bytes per lane: forward, 16-bit storage
+            assert p.vec in ((1, 2, 4, 8) if wide else (1, 2, 4)) and D % p.vec == 0 and align % p.vec == 0, what
             assert p.steps in (4, 8) and p.threads in (256, 512, 1024), what
             assert 1 <= (1 << p.g_log2) <= p.threads and p.strip_cols == p.vec << p.g_log2, what
             assert p.seg_len == p.steps * (p.threads >> p.g_log2) and p.seg_len % p.ckpt_stride == 0, what

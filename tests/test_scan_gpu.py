@@ -183,6 +183,55 @@ def test_lds_resident_operands_and_register_path_agree(gpu, dtype, shape, g_log2
         assert_close(k, got32[k], ref32[k], TOL[dtype])
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+@pytest.mark.parametrize("g_log2", [5, 4, 2], ids=["rows32", "rows16", "rows4"])
+@pytest.mark.parametrize("shape", [(2, 700, 512), (2, 1100, 264), (1, 97, 256), (1, 2100, 40)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_forward_with_sixteen_bytes_per_lane(gpu, dtype, shape, g_log2):
+    # The forward over 16-bit storage that large launches take by themselves (8 columns = 16 bytes per lane, c
+    # loaded straight into LDS), forced here onto small shapes: ragged last tiles, a partial last strip, several
+    # clusters per chain, rows narrower than a wavefront, y in the operands' storage and in fp32, the full fp32
+    # state, rows off a 16-byte boundary (c then goes through registers), and its saved states feeding the
+    # (unchanged) backward.
+    B, L, D = shape
+    x, a, b, c, dy = make_inputs(shape, dtype=dtype, seed=33)
+    ref = oracle_all(x, a, b, c, dy)
+    tune = (g_log2 + 1) | (8 << 16)
+    bwd_tune = 7 | (8 << 8)      # the backward at its usual 64-lane rows: saved states 32 steps apart
+    plan = hip_scan.make_plan(B, L, D, dtype, dtype, _lib.QSSM_FORWARD, 8, 32, tune)
+    assert (plan.vec, plan.steps, plan.threads, plan.g_log2) == (8, 8, 256, g_log2)
+
+    def run(place, out_dtype=dtype, gy=dy, keep_h=False):
+        ops = [place(t) for t in (x, a, b, c)]
+        y, h, ckpt, stride = hip_scan.scan_forward(*ops, out_dtype=out_dtype, want_h=keep_h, want_ckpt=not keep_h,
+                                                   tune=tune, bwd_tune=bwd_tune)
+        assert stride == 32 or keep_h
+        dx, da, db, dc = hip_scan.scan_backward(*ops, place(gy), h=h, ckpt=ckpt, ckpt_stride=stride, tune=bwd_tune)
+        assert hip_scan.workspace_status() == 0
+        return {k: v.cpu() for k, v in zip(("y", "dx", "da", "db", "dc"), (y, dx, da, db, dc))}, h
+
+    def aligned(t):
+        return t.to(gpu).contiguous()
+
+    def shifted(t):  # same values, every row 16 bytes off a 32-byte boundary but 8 elements apart in alignment
+        buf = torch.zeros(B, L, D + 16, dtype=t.dtype, device=gpu)
+        buf[:, :, 8:8 + D] = t.to(gpu)
+        return buf[:, :, 8:8 + D]
+
+    _check_all(run(aligned)[0], ref, TOL[dtype])
+    got, h = run(aligned, keep_h=True)
+    _check_all(got, ref, TOL[dtype])
+    h64, _ = oracle.forward_f64(x, a, b, c)
+    assert_close("h", h.cpu(), h64, 1e-5)
+    _check_all(run(shifted)[0], ref, TOL[dtype])
+    x32, a32, b32, c32, dy32 = make_inputs(shape, dtype=dtype, seed=33, out_dtype=torch.float32)
+    got32, _ = run(aligned, out_dtype=torch.float32, gy=dy32)
+    ref32 = oracle_all(x32, a32, b32, c32, dy32)
+    assert_close("y", got32["y"], ref32["y"], 1e-5)
+    for k in ("dx", "da", "db", "dc"):
+        assert_close(k, got32[k], ref32[k], TOL[dtype])
+
+
 def test_mixed_operand_dtypes_and_unbuilt_output_dtype(gpu):
     x, a, b, c, dy = make_inputs((2, 130, 8), seed=2)
     a16, c16 = a.to(torch.float16), c.to(torch.bfloat16)
