@@ -362,6 +362,57 @@ QSSM_API int qssm_gates_backward(const void* g_a, const void* g_x, const void* g
                         int64_t rows, int32_t S, int32_t in_dtype, int32_t out_dtype, void* stream);
 
 /*
+ * The scan with the layer's gate activations inside it (quick_ssm/layers.py:76-104 as one launch each way): the
+ * operands are the five projection outputs, [B, L, S] with batch and time strides in elements (so they may be
+ * column slices of one wide GEMM output), stored as f16 or bf16, and
+ *     a = sigmoid(A_pre), x = B_in, b = sigmoid(D_pre), c = silu(Ca) * Cb
+ * are formed in registers, rounded to the projections' storage type exactly where the layer's cast to its compute
+ * dtype rounds them (layers.py:85-88); then h(t) = a h(t-1) + b x, y = c h as in qssm_scan_forward.  The backward
+ * returns the projections' gradients directly,
+ *     dA_pre = da a (1 - a), dB_in = dx, dD_pre = db b (1 - b), dCa = dc Cb s (1 + Ca (1 - s)), dCb = dc Ca s,
+ * s = sigmoid(Ca), with da, db, dc rounded to the storage type as qssm_scan_backward stores them.  The tensors a,
+ * x, b, c and their gradients never reach HBM: 12 instead of 30 bytes per element forward and 22 instead of 46
+ * backward for bf16.
+ *   - Plans come from qssm_plan_scan_gated (one geometry: 4 columns x 8 steps per lane, 256 lanes); shapes it
+ *     refuses (D < 128, rows not 16-byte aligned, fp32 projections) take qssm_gates_* + qssm_scan_*.
+ *   - ckpt, control, workspace, epoch: as for qssm_scan_forward / qssm_scan_backward; the backward needs the saved
+ *     states (the checkpoint=True case) and y / dy stored as the projections are (forward: or as f32).
+ * Replaces SSM.forward's elementwise chain and scan call, quick_ssm/layers.py:76-104, and what autograd records
+ * for them.
+ */
+QSSM_API int qssm_plan_scan_gated(int32_t B, int32_t L, int32_t D, int32_t dtype, int32_t out_dtype,
+                         int32_t direction, int32_t align_elems, int32_t ckpt_stride, qssm_plan* plan);
+
+QSSM_API int qssm_scan_gated_forward(const qssm_plan* plan,
+                            const void* A_pre, qssm_strides sA,
+                            const void* B_in, qssm_strides sB,
+                            const void* Ca, qssm_strides sCa,
+                            const void* Cb, qssm_strides sCb,
+                            const void* D_pre, qssm_strides sD,
+                            void* y, qssm_strides sy,
+                            float* ckpt,
+                            void* control, uint64_t control_size,
+                            void* workspace, uint64_t workspace_bytes, uint32_t epoch,
+                            void* stream);
+
+QSSM_API int qssm_scan_gated_backward(const qssm_plan* plan,
+                             const void* A_pre, qssm_strides sA,
+                             const void* B_in, qssm_strides sB,
+                             const void* Ca, qssm_strides sCa,
+                             const void* Cb, qssm_strides sCb,
+                             const void* D_pre, qssm_strides sD,
+                             const void* dy, qssm_strides sdy,
+                             const float* ckpt,
+                             void* dA_pre, qssm_strides sdA,
+                             void* dB_in, qssm_strides sdB,
+                             void* dCa, qssm_strides sdCa,
+                             void* dCb, qssm_strides sdCb,
+                             void* dD_pre, qssm_strides sdD,
+                             void* control, uint64_t control_size,
+                             void* workspace, uint64_t workspace_bytes, uint32_t epoch,
+                             void* stream);
+
+/*
  * RMSNorm of the SSM layer over the last axis: y = x * weight / sqrt(mean(x^2) + eps).
  * x is [rows, H] with row stride ld_x elements, weight [H], y [rows, H] contiguous, all stored as `dtype`
  * (f32, f16 or bf16); fp32 arithmetic, one rounding per result.  `rstd` ([rows] fp32, or NULL) receives

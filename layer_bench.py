@@ -13,6 +13,7 @@ algorithmic bytes: what it must read and write once.
     gates forward     rows x S x (5 s_p + 4 s_c)    five projections in, four operands out
     gates backward    rows x S x (4 s_c + 4 s_p + 5 s_p)
     scan forward      rows x S x (4 s_c + s_y)      scan backward  rows x S x (8 s_c + s_y)
+    gated scan        rows x S x 6 s_p forward (five projections in, y out), 11 s_p backward (16-bit projections)
 
 One JSON line is printed; `layer_step_ms` is forward + backward of the whole layer (GEMMs included)
 through autograd, with the fused passes and, beside it, with the same formulas as separate torch ops.
@@ -134,6 +135,32 @@ def main() -> int:
             record("scan_backward", us, rows * S * (8 * sc + sp))
         del ops, gy, ckpt
 
+    # ---- the gated scan: projection outputs in, y / projection gradients out, one launch each way -----------
+    from quick_ssm_amd import gated_scan
+
+    z = [torch.randn(B, L, S, device=dev).mul_(1.5).to(pdt) for _ in range(5)]
+    z[0] += 3.0
+    if gated_scan.supported(z, cdt, pdt):
+        gy = torch.randn(B, L, S, device=dev).to(pdt)
+        leaves = [t.requires_grad_(True) for t in z]
+        with torch.no_grad():
+            us = _time_us(torch, lambda: gated_scan.gated_scan(*leaves, out_dtype=pdt), args.steps, args.warmup)
+        record("gated_scan_forward", us, rows * S * (5 * sp + sp))
+
+        def fwd_bwd():
+            for t in leaves:
+                t.grad = None
+            gated_scan.gated_scan(*leaves, out_dtype=pdt).backward(gy)
+
+        both = _time_us(torch, fwd_bwd, args.steps, args.warmup)
+        record("gated_scan_backward", both - us, rows * S * (5 * sp + sp + 5 * sp))
+        passes["non_gemm_bytes_per_element"] = {
+            "two_pass": {"forward": 5 * sp + 4 * sc + 4 * sc + sp, "backward": 8 * sc + sp + 4 * sc + 9 * sp},
+            "gated": {"forward": 6 * sp, "backward": 11 * sp},
+        }
+        del gy, leaves
+    del z
+
     # ---- the whole layer step, fused passes against separate torch ops ---------------------------------
     layer = layers.SSM(H, args.mult, dtype=pdt, device=dev, compute_dtype=cdt)
     inp = torch.randn(B, L, H, device=dev).to(pdt).requires_grad_(True)
@@ -144,18 +171,26 @@ def main() -> int:
         layer(inp).sum().backward()
 
     fused_ms = _time_us(torch, step, max(3, args.steps // 2), 2) / 1e3
-    keep = layers.gate_prologue, layers.rms_norm
-    layers.gate_prologue, layers.rms_norm = gates.gates_reference, norm.rms_norm_reference
+    # the same step with the activations in a pass of their own (what every layer took before the gated scan)
+    keep_supported = gated_scan.supported
+    gated_scan.supported = lambda *a, **k: False
     try:
-        torch_ms = _time_us(torch, step, max(3, args.steps // 2), 2) / 1e3
+        two_pass_ms = _time_us(torch, step, max(3, args.steps // 2), 2) / 1e3
+        keep = layers.gate_prologue, layers.rms_norm
+        layers.gate_prologue, layers.rms_norm = gates.gates_reference, norm.rms_norm_reference
+        try:
+            torch_ms = _time_us(torch, step, max(3, args.steps // 2), 2) / 1e3
+        finally:
+            layers.gate_prologue, layers.rms_norm = keep
     finally:
-        layers.gate_prologue, layers.rms_norm = keep
+        gated_scan.supported = keep_supported
 
     print(json.dumps({
         "config": {"batch": B, "length": L, "hidden": H, "state": S, "param_dtype": args.param_dtype,
                    "compute_dtype": args.compute_dtype},
         "passes": passes,
-        "layer_step_ms": {"fused_passes": fused_ms, "torch_ops_for_norm_and_gates": torch_ms},
+        "layer_step_ms": {"fused_passes": fused_ms, "gates_in_a_pass_of_their_own": two_pass_ms,
+                          "torch_ops_for_norm_and_gates": torch_ms},
         "workspace_status": hip_scan.workspace_status(),
     }), flush=True)
     return 0

@@ -35,6 +35,9 @@ EXPORTED_SYMBOLS = (
     "qssm_scan_forward_static",
     "qssm_scan_forward_call",
     "qssm_scan_backward_call",
+    "qssm_plan_scan_gated",
+    "qssm_scan_gated_forward",
+    "qssm_scan_gated_backward",
     "qssm_gates_forward",
     "qssm_gates_backward",
     "qssm_rmsnorm_forward",
@@ -157,6 +160,16 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.qssm_scan_backward_carry.argtypes = (
         [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, vp, vp] + [vp, Strides] * 4
         + [vp, u64, vp, u64, ctypes.c_uint32, vp]
+    )
+    lib.qssm_plan_scan_gated.restype = ctypes.c_int
+    lib.qssm_plan_scan_gated.argtypes = [i32] * 8 + [ctypes.POINTER(Plan)]
+    lib.qssm_scan_gated_forward.restype = ctypes.c_int
+    lib.qssm_scan_gated_forward.argtypes = (
+        [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, u64, vp, u64, ctypes.c_uint32, vp]
+    )
+    lib.qssm_scan_gated_backward.restype = ctypes.c_int
+    lib.qssm_scan_gated_backward.argtypes = (
+        [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, Strides] * 5 + [vp, u64, vp, u64, ctypes.c_uint32, vp]
     )
     i64 = ctypes.c_int64
     lib.qssm_gates_forward.restype = ctypes.c_int

@@ -14,8 +14,6 @@
 
 namespace qssm {
 
-__device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
-
 template <typename T, int V>
 __device__ __forceinline__ void load_f32(const void* base, int64_t elem_off, float* out) {
   const Words<T, V> w = load_stream<T, V>(reinterpret_cast<const char*>(base) + elem_off * (int64_t)sizeof(T), 0u);

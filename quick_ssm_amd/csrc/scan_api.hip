@@ -174,11 +174,26 @@ static void fill_geometry(Geometry* g, const qssm_plan* pl, void* control, void*
 
 using namespace qssm;
 
+// What a gated launch has beyond a plain one: the second factor of c and, backwards, where its gradient goes.
+struct GateExtras {
+  const void* c2;
+  qssm_strides sc2;
+  void* dc2;
+  qssm_strides sdc2;
+};
+
 static int forward_launch(const qssm_plan* plan, const void* x, qssm_strides sx, const void* a, qssm_strides sa,
                           const void* b, qssm_strides sb, const void* c, qssm_strides sc, void* y, qssm_strides sy,
                           float* h_out, qssm_strides sh, float* ckpt, const float* h_init, float* h_final,
                           void* control, uint64_t control_size, void* workspace, uint64_t workspace_bytes,
-                          uint32_t epoch, unsigned count_reset_at, void* stream);
+                          uint32_t epoch, unsigned count_reset_at, void* stream, const GateExtras* gate = nullptr);
+static int backward_launch(const qssm_plan* plan, const void* x, qssm_strides sx, const void* a, qssm_strides sa,
+                           const void* b, qssm_strides sb, const void* c, qssm_strides sc, const void* dy,
+                           qssm_strides sdy, const float* h, qssm_strides sh, const float* ckpt, const float* h_init,
+                           const float* dh_final, float* dh_init, void* dx, qssm_strides sdx, void* da,
+                           qssm_strides sda, void* db, qssm_strides sdb, void* dc, qssm_strides sdc, void* control,
+                           uint64_t control_size, void* workspace, uint64_t workspace_bytes, uint32_t epoch,
+                           void* stream, const GateExtras* gate = nullptr);
 
 extern "C" {
 
@@ -189,6 +204,28 @@ const char* qssm_error_string(void) { return g_err; }
 int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int32_t out_dtype, int32_t direction,
                    int32_t align_elems, int32_t ckpt_stride, qssm_plan* plan) {
   return qssm_plan_scan_tuned(B, L, D, in_dtype, out_dtype, direction, align_elems, ckpt_stride, 0, plan);
+}
+
+// The gated kernels exist in one shape: 4 columns (8 bytes of 16-bit storage) and 8 steps per lane, 256 lanes,
+// rows of 64 or 32 lanes, clusters of at most two tiles (the backward's three LDS-resident operands leave LDS
+// for no more neighbour maps).
+static const int32_t kGatedTune = (8 << 8) | (4 << 16) | (1 << 24);
+int qssm_plan_scan_gated(int32_t B, int32_t L, int32_t D, int32_t dtype, int32_t out_dtype, int32_t direction,
+                         int32_t align_elems, int32_t ckpt_stride, qssm_plan* plan) {
+  if (dtype_size(dtype) != 2) return fail(QSSM_EINVAL, "the gated scan is built for 16-bit projections");
+  if (D % 4 != 0 || align_elems % 8 != 0 || D < 128)
+    return fail(QSSM_EALIGN, "the gated scan needs D >= 128, a multiple of 4, and 16-byte aligned rows");
+  int rc = qssm_plan_scan_tuned(B, L, D, dtype, out_dtype, direction, align_elems, ckpt_stride, kGatedTune, plan);
+  if (rc != 0 || B == 0 || L == 0) return rc;
+  int g_log2 = plan->g_log2 > 6 ? 6 : (plan->g_log2 < 5 ? 5 : plan->g_log2);
+  if (g_log2 != plan->g_log2 || plan->cluster > 2)   // same strips, more hand-overs, less LDS
+    rc = qssm_plan_scan_tuned(B, L, D, dtype, out_dtype, direction, align_elems, ckpt_stride,
+                              kGatedTune | (g_log2 + 1) | ((plan->cluster > 2 ? 2 : 0) << 28), plan);
+  if (rc != 0) return rc;
+  if (plan->vec != 4 || plan->steps != 8 || plan->threads != 256 || (plan->g_log2 != 6 && plan->g_log2 != 5) ||
+      plan->cluster > 2)
+    return fail(QSSM_EINVAL, "no gated geometry for this shape");
+  return 0;
 }
 
 int qssm_plan_scan_tuned(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int32_t out_dtype, int32_t direction,
@@ -425,7 +462,7 @@ static int forward_launch(const qssm_plan* plan, const void* x, qssm_strides sx,
                           const void* b, qssm_strides sb, const void* c, qssm_strides sc, void* y, qssm_strides sy,
                           float* h_out, qssm_strides sh, float* ckpt, const float* h_init, float* h_final,
                           void* control, uint64_t control_size, void* workspace, uint64_t workspace_bytes,
-                          uint32_t epoch, unsigned count_reset_at, void* stream) {
+                          uint32_t epoch, unsigned count_reset_at, void* stream, const GateExtras* gate) {
   int rc = check_plan(plan, QSSM_FORWARD);
   if (rc != 0) return rc;
   if (plan->B == 0 || plan->L == 0 || plan->D == 0) return 0;
@@ -471,7 +508,17 @@ static int forward_launch(const qssm_plan* plan, const void* x, qssm_strides sx,
                   ((uintptr_t)c) % 16 == 0 && (sc.b * es) % 16 == 0 && (sc.l * es) % 16 == 0 &&
                   lds + fwd_c_lds_bytes(plan->threads, plan->steps, v * es) <= (size_t)kMaxLdsBytes;
   if (c_in_lds) lds += fwd_c_lds_bytes(plan->threads, plan->steps, v * es);
-  if (!fn(args, plan->vec, plan->steps, plan->threads, c_in_lds, grid, lds, (hipStream_t)stream))
+  args.c2 = nullptr; args.c2_sb = args.c2_sl = 0;
+  if (gate != nullptr) {
+    // Ca and Cb both go through LDS: the same conditions again for Cb, and room for the second array
+    if (!c_in_lds || !narrow_rows || plan->threads != 256 || gate->c2 == nullptr || ((uintptr_t)gate->c2) % 16 != 0 ||
+        (gate->sc2.b * es) % 16 != 0 || (gate->sc2.l * es) % 16 != 0 || !tile_span_ok(plan, gate->c2, gate->sc2.b, gate->sc2.l, es) ||
+        lds + fwd_c_lds_bytes(plan->threads, plan->steps, v * es) > (size_t)kMaxLdsBytes)
+      return fail(QSSM_EALIGN, "gated scan needs a plan of qssm_plan_scan_gated, y, and Ca, Cb with 16-byte aligned rows");
+    lds += fwd_c_lds_bytes(plan->threads, plan->steps, v * es);
+    args.c2 = gate->c2; args.c2_sb = gate->sc2.b; args.c2_sl = gate->sc2.l;
+  }
+  if (!fn(args, plan->vec, plan->steps, plan->threads, c_in_lds, gate != nullptr, grid, lds, (hipStream_t)stream))
     return fail(QSSM_EINVAL, "no forward kernel for vec=%d steps=%d threads=%d", plan->vec, plan->steps, plan->threads);
   if (epoch == 0 && plan->n_seg > 1)
     hipLaunchKernelGGL(count_launch_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream,
@@ -500,6 +547,19 @@ int qssm_scan_backward_carry(const qssm_plan* plan, const void* x, qssm_strides 
                              void* da, qssm_strides sda, void* db, qssm_strides sdb, void* dc, qssm_strides sdc,
                              void* control, uint64_t control_size, void* workspace, uint64_t workspace_bytes,
                              uint32_t epoch, void* stream) {
+  return backward_launch(plan, x, sx, a, sa, b, sb, c, sc, dy, sdy, h, sh, ckpt, h_init, dh_final, dh_init, dx, sdx, da,
+                         sda, db, sdb, dc, sdc, control, control_size, workspace, workspace_bytes, epoch, stream);
+}
+
+}  // extern "C"
+
+static int backward_launch(const qssm_plan* plan, const void* x, qssm_strides sx, const void* a, qssm_strides sa,
+                           const void* b, qssm_strides sb, const void* c, qssm_strides sc, const void* dy,
+                           qssm_strides sdy, const float* h, qssm_strides sh, const float* ckpt, const float* h_init,
+                           const float* dh_final, float* dh_init, void* dx, qssm_strides sdx, void* da,
+                           qssm_strides sda, void* db, qssm_strides sdb, void* dc, qssm_strides sdc, void* control,
+                           uint64_t control_size, void* workspace, uint64_t workspace_bytes, uint32_t epoch,
+                           void* stream, const GateExtras* gate) {
   int rc = check_plan(plan, QSSM_BACKWARD);
   if (rc != 0) return rc;
   if (plan->B == 0 || plan->L == 0 || plan->D == 0) return 0;
@@ -551,13 +611,57 @@ int qssm_scan_backward_carry(const qssm_plan* plan, const void* x, qssm_strides 
                    ((uintptr_t)dy) % 16 == 0 && (sdy.b * os) % 16 == 0 && (sdy.l * os) % 16 == 0 &&
                    lds + bwd_cg_lds_bytes(plan->threads, plan->steps) <= (size_t)kMaxLdsBytes;
   if (cg_in_lds) lds += bwd_cg_lds_bytes(plan->threads, plan->steps);
-  if (!fn(args, plan->vec, plan->steps, plan->threads, cg_in_lds, grid, lds, (hipStream_t)stream))
+  args.c2 = nullptr; args.c2_sb = args.c2_sl = 0; args.dc2 = nullptr; args.dc2_sb = args.dc2_sl = 0;
+  if (gate != nullptr) {
+    // Ca, Cb and dy all go through LDS: the same conditions again for Cb, and room for the third array
+    const size_t one = bwd_cg_lds_bytes(plan->threads, plan->steps) / 2;
+    if (!cg_in_lds || h != nullptr || gate->c2 == nullptr || ((uintptr_t)gate->c2) % 16 != 0 || (gate->sc2.b * es) % 16 != 0 ||
+        (gate->sc2.l * es) % 16 != 0 || !tile_span_ok(plan, gate->c2, gate->sc2.b, gate->sc2.l, es) ||
+        !aligned_to(gate->dc2, gate->sdc2.b, gate->sdc2.l, es, v) || !tile_span_ok(plan, gate->dc2, gate->sdc2.b, gate->sdc2.l, es) ||
+        lds + one > (size_t)kMaxLdsBytes)
+      return fail(QSSM_EALIGN, "gated scan needs a plan of qssm_plan_scan_gated, 16-bit dy, saved states, and Ca, Cb, dy with "
+                               "16-byte aligned rows");
+    lds += one;
+    args.c2 = gate->c2; args.c2_sb = gate->sc2.b; args.c2_sl = gate->sc2.l;
+    args.dc2 = gate->dc2; args.dc2_sb = gate->sdc2.b; args.dc2_sl = gate->sdc2.l;
+  }
+  if (!fn(args, plan->vec, plan->steps, plan->threads, cg_in_lds, gate != nullptr, grid, lds, (hipStream_t)stream))
     return fail(QSSM_EINVAL, "no backward kernel for vec=%d steps=%d threads=%d", plan->vec, plan->steps, plan->threads);
   if (epoch == 0 && plan->n_seg > 1)
     hipLaunchKernelGGL(count_launch_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream,
                        (unsigned*)((char*)control + kLaunchCountOffset), kCountWrapAt);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : hip_fail(e, "scan_bwd_kernel launch");
+}
+
+extern "C" {
+
+int qssm_scan_gated_forward(const qssm_plan* plan, const void* A_pre, qssm_strides sA, const void* B_in, qssm_strides sB,
+                            const void* Ca, qssm_strides sCa, const void* Cb, qssm_strides sCb, const void* D_pre,
+                            qssm_strides sD, void* y, qssm_strides sy, float* ckpt, void* control,
+                            uint64_t control_size, void* workspace, uint64_t workspace_bytes, uint32_t epoch,
+                            void* stream) {
+  if (A_pre == nullptr || B_in == nullptr || Ca == nullptr || Cb == nullptr || D_pre == nullptr || y == nullptr)
+    return fail(QSSM_EINVAL, "the five projection outputs and y must not be NULL");
+  const GateExtras gate{Cb, sCb, nullptr, qssm_strides{0, 0}};
+  return forward_launch(plan, B_in, sB, A_pre, sA, D_pre, sD, Ca, sCa, y, sy, nullptr, qssm_strides{0, 0}, ckpt, nullptr,
+                        nullptr, control, control_size, workspace, workspace_bytes, epoch, kCountWrapAt, stream, &gate);
+}
+
+int qssm_scan_gated_backward(const qssm_plan* plan, const void* A_pre, qssm_strides sA, const void* B_in,
+                             qssm_strides sB, const void* Ca, qssm_strides sCa, const void* Cb, qssm_strides sCb,
+                             const void* D_pre, qssm_strides sD, const void* dy, qssm_strides sdy, const float* ckpt,
+                             void* dA_pre, qssm_strides sdA, void* dB_in, qssm_strides sdB, void* dCa,
+                             qssm_strides sdCa, void* dCb, qssm_strides sdCb, void* dD_pre, qssm_strides sdD,
+                             void* control, uint64_t control_size, void* workspace, uint64_t workspace_bytes,
+                             uint32_t epoch, void* stream) {
+  if (A_pre == nullptr || B_in == nullptr || Ca == nullptr || Cb == nullptr || D_pre == nullptr || dy == nullptr ||
+      ckpt == nullptr)
+    return fail(QSSM_EINVAL, "the five projection outputs, dy and the saved states must not be NULL");
+  const GateExtras gate{Cb, sCb, dCb, sdCb};
+  return backward_launch(plan, B_in, sB, A_pre, sA, D_pre, sD, Ca, sCa, dy, sdy, nullptr, qssm_strides{0, 0}, ckpt, nullptr,
+                         nullptr, nullptr, dB_in, sdB, dA_pre, sdA, dD_pre, sdD, dCa, sdCa, control, control_size,
+                         workspace, workspace_bytes, epoch, stream, &gate);
 }
 
 // Widest lane vector (4, 2 or 1 elements) every listed tensor allows.

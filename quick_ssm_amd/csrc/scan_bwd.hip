@@ -27,8 +27,16 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // sweeps that use them: 32 VGPRs fewer across the tile's whole life, which is one more resident
 // workgroup per SIMD.  Needs 64 lanes per row and 8 bytes per lane in both tensors, so that one
 // wavefront-wide 16-byte-per-lane load covers two rows of the strip.
-template <typename Tin, typename Tout, int VEC, int T, int NTH, bool CLDS>
+//
+// GATED: the operands are the SSM layer's projection outputs (quick_ssm/layers.py:76-88) and both the gate
+// activations and their derivatives happen here: a = sigmoid(A_pre), b = sigmoid(D_pre) replace their
+// pre-activations in registers, c = silu(Ca) * Cb is formed from two LDS-resident operands where it is used, and
+// the last sweep turns the scan's gradients (rounded to the storage type, as the scan stores them) into the
+// projections' gradients dA_pre = da a (1 - a), dB_in = dx, dD_pre = db b (1 - b),
+// dCa = dc Cb s (1 + Ca (1 - s)), dCb = dc Ca s with s = sigmoid(Ca): no gradient of a, x, b, c ever exists in HBM.
+template <typename Tin, typename Tout, int VEC, int T, int NTH, bool CLDS, bool GATED>
 __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
+  static_assert(!GATED || CLDS, "gated scan: Ca, Cb and dy through LDS");
   static_assert(!CLDS || (sizeof(Tin) * VEC == 8 && sizeof(Tout) * VEC == 8 && T % 2 == 0),
                 "LDS-resident c and dy: 8 bytes per lane, even step count");
   extern __shared__ __align__(16) float lds[];
@@ -48,6 +56,7 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   int* sSeg = reinterpret_cast<int*>(sE + cols);
   char* sC = reinterpret_cast<char*>(sSeg) + 16 + ((int)threadIdx.x >> 6) * (T * 512);  // CLDS: this wave's [T rows][512 bytes] of c
   char* sG = sC + (NTH / 64) * (T * 512);                                  // and of dy
+  char* sC2 = sG + (NTH / 64) * (T * 512);                                 // GATED: and of Cb (sC then holds Ca)
   // Where step i of this lane sits in its wavefront's LDS block: the loads that fill it deposit 1024 bytes per
   // instruction in lane order, i.e. per pair of steps [group in wavefront][step parity][G * 8 bytes].
   const int lds_lane = (((int)threadIdx.x & 63) >> g.g_log2) * (G * 16) + ((int)threadIdx.x & (G - 1)) * 8;
@@ -88,6 +97,8 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
             store_stream<Tin, VEC>((char*)p.db + ((int64_t)pbi * p.db_sb + (int64_t)t * p.db_sl + pd) * (int64_t)sizeof(Tin), 0u, nanv);
           if (p.dc != nullptr)
             store_stream<Tin, VEC>((char*)p.dc + ((int64_t)pbi * p.dc_sb + (int64_t)t * p.dc_sl + pd) * (int64_t)sizeof(Tin), 0u, nanv);
+          if (GATED && p.dc2 != nullptr)
+            store_stream<Tin, VEC>((char*)p.dc2 + ((int64_t)pbi * p.dc2_sb + (int64_t)t * p.dc2_sl + pd) * (int64_t)sizeof(Tin), 0u, nanv);
         }
       }
       if (p.dh_init != nullptr && pseg == 0 && (tid >> g.g_log2) == 0 && pd < g.D)
@@ -118,6 +129,8 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   const uint32_t bo = (uint32_t)((j * T * (int)p.b_sl + dl) * (int)sizeof(Tin)), bs = (uint32_t)p.b_sl * sizeof(Tin);
   const uint32_t co = (uint32_t)((j * T * (int)p.c_sl + dl) * (int)sizeof(Tin)), cs = (uint32_t)p.c_sl * sizeof(Tin);
   const uint32_t go = (uint32_t)((j * T * (int)p.dy_sl + dl) * (int)sizeof(Tout)), gs = (uint32_t)p.dy_sl * sizeof(Tout);
+  const char* c2b = GATED ? (const char*)p.c2 + ((int64_t)bi * p.c2_sb + (int64_t)t_tile * p.c2_sl + col0) * (int64_t)sizeof(Tin) : nullptr;
+  const uint32_t c2o = GATED ? (uint32_t)((j * T * (int)p.c2_sl + dl) * (int)sizeof(Tin)) : 0u, c2s = GATED ? (uint32_t)p.c2_sl * sizeof(Tin) : 0u;
   const float* hp = p.h + (int64_t)bi * p.h_sb + (int64_t)t0 * p.h_sl + d;
 
   // ---- ask for the neighbours' words first: they are looked at once the answers are back ------
@@ -159,6 +172,12 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
       for (int k = 0; k < T / 2; ++k) {
         __builtin_amdgcn_global_load_lds((global_ptr_t)(csrc + (uint32_t)(2 * k) * cs), (lds_ptr_t)(sC + k * 1024), 16, 0, 2);
         __builtin_amdgcn_global_load_lds((global_ptr_t)(gsrc + (uint32_t)(2 * k) * gs), (lds_ptr_t)(sG + k * 1024), 16, 0, 2);
+      }
+      if constexpr (GATED) {
+        const char* c2src = c2b + (uint32_t)(j * T + half) * c2s + (uint32_t)piece * 16u;
+#pragma unroll
+        for (int k = 0; k < T / 2; ++k)
+          __builtin_amdgcn_global_load_lds((global_ptr_t)(c2src + (uint32_t)(2 * k) * c2s), (lds_ptr_t)(sC2 + k * 1024), 16, 0, 2);
       }
     } else {
 #pragma unroll
@@ -210,6 +229,11 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
         }
         *reinterpret_cast<Words<Tin, VEC>*>(sC + lds_row(i) + lds_lane) = cw;
         *reinterpret_cast<Words<Tout, VEC>*>(sG + lds_row(i) + lds_lane) = gw;
+        if constexpr (GATED) {
+          Words<Tin, VEC> cw2 = fill_words<Tin, VEC>(false);
+          if (dok && t0 + i < g.L) cw2 = load_stream<Tin, VEC>(c2b, c2o + i * c2s);
+          *reinterpret_cast<Words<Tin, VEC>*>(sC2 + lds_row(i) + lds_lane) = cw2;
+        }
       }
     }
   }
@@ -272,10 +296,25 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
 
   // ---- sweep 1: fold this lane's T steps into the forward and the reverse affine map ----------
   float A[VEC], Xf[VEC], Xe[VEC];
+  Words<Tin, VEC> za[GATED ? T : 1], zd[GATED ? T : 1];   // GATED: A_pre and D_pre as loaded
 #pragma unroll
   for (int v = 0; v < VEC; ++v) { A[v] = 1.0f; Xf[v] = 0.0f; Xe[v] = 0.0f; }
 #pragma unroll
   for (int i = 0; i < T; ++i) {
+    if constexpr (GATED) {
+      // The pre-activations stay beside the gates they turn into: the last sweep wants the derivatives
+      // a (1 - a), b (1 - b) of the unrounded gates (1 - a loses most of its digits when a, close to one, is
+      // first rounded to 16 bits).  Steps past L and columns past D hold the identity (a = 1, b = 0) and keep it.
+      za[i] = ra[i];
+      zd[i] = rb[i];
+      if (tile_full || (dok && t0 + i < g.L)) {
+        float ga[VEC], gb[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) { ga[v] = sigmoid_f(elem(ra[i], v)); gb[v] = sigmoid_f(elem(rb[i], v)); }
+        ElemBits<Tin>::template set<VEC>(ra[i], ga);
+        ElemBits<Tin>::template set<VEC>(rb[i], gb);
+      }
+    }
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
       const float av = elem(ra[i], v);
@@ -297,6 +336,13 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
     } else {
       cw = rc[i];
       gw = rg[i];
+    }
+    if constexpr (GATED) {
+      const Words<Tin, VEC> cw2 = *reinterpret_cast<const Words<Tin, VEC>*>(sC2 + lds_row(i) + lds_lane);
+      float gc[VEC];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) { const float ca = elem(cw, v); gc[v] = ca * sigmoid_f(ca) * elem(cw2, v); }
+      ElemBits<Tin>::template set<VEC>(cw, gc);
     }
 #pragma unroll
     for (int v = 0; v < VEC; ++v)
@@ -436,9 +482,11 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   const uint32_t dao = (uint32_t)((j * T * (int)p.da_sl + dl) * (int)sizeof(Tin)), das = (uint32_t)p.da_sl * sizeof(Tin);
   const uint32_t dbo = (uint32_t)((j * T * (int)p.db_sl + dl) * (int)sizeof(Tin)), dbs = (uint32_t)p.db_sl * sizeof(Tin);
   const uint32_t dco = (uint32_t)((j * T * (int)p.dc_sl + dl) * (int)sizeof(Tin)), dcs = (uint32_t)p.dc_sl * sizeof(Tin);
+  char* dc2b = GATED ? (char*)p.dc2 + ((int64_t)bi * p.dc2_sb + (int64_t)t_tile * p.dc2_sl + col0) * (int64_t)sizeof(Tin) : nullptr;
+  const uint32_t dc2o = GATED ? (uint32_t)((j * T * (int)p.dc2_sl + dl) * (int)sizeof(Tin)) : 0u, dc2s = GATED ? (uint32_t)p.dc2_sl * sizeof(Tin) : 0u;
 #pragma unroll
   for (int i = T - 1; i >= 0; --i) {
-    float vdx[VEC], vda[VEC], vdb[VEC], vdc[VEC];
+    float vdx[VEC], vda[VEC], vdb[VEC], vdc[VEC], vdc2[VEC];
     Words<Tin, VEC> cw;
     Words<Tout, VEC> gw;
     if (CLDS) {
@@ -447,6 +495,19 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
     } else {
       cw = rc[i];
       gw = rg[i];
+    }
+    float zca[VEC], zcb[VEC], sg[VEC];   // GATED: Ca, Cb and sigmoid(Ca) of this step
+    if constexpr (GATED) {
+      const Words<Tin, VEC> cw2 = *reinterpret_cast<const Words<Tin, VEC>*>(sC2 + lds_row(i) + lds_lane);
+      float gc[VEC];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        zca[v] = elem(cw, v);
+        zcb[v] = elem(cw2, v);
+        sg[v] = sigmoid_f(zca[v]);
+        gc[v] = zca[v] * sg[v] * zcb[v];
+      }
+      ElemBits<Tin>::template set<VEC>(cw, gc);
     }
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
@@ -459,11 +520,28 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
       vda[v] = hm * dH;
       E[v] = elem(ra[i], v) * dH;
     }
+    if constexpr (GATED) {
+      // the scan's gradients as it would have stored them, then through the activations' derivatives
+      round_through<Tin, VEC>(vda);
+      round_through<Tin, VEC>(vdb);
+      round_through<Tin, VEC>(vdc);
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        const float av = sigmoid_f(elem(za[i], v)), bv = sigmoid_f(elem(zd[i], v));
+        vda[v] = vda[v] * av * (1.0f - av);
+        vdb[v] = vdb[v] * bv * (1.0f - bv);
+        vdc2[v] = vdc[v] * zca[v] * sg[v];
+        vdc[v] = vdc[v] * zcb[v] * sg[v] * (1.0f + zca[v] * (1.0f - sg[v]));
+      }
+    }
     if (tile_full || (dok && t0 + i < g.L)) {
       if (p.dx != nullptr) store_stream<Tin, VEC>(dxb, dxo + i * dxs, vdx);
       if (p.da != nullptr) store_stream<Tin, VEC>(dab, dao + i * das, vda);
       if (p.db != nullptr) store_stream<Tin, VEC>(dbb, dbo + i * dbs, vdb);
       if (p.dc != nullptr) store_stream<Tin, VEC>(dcb, dco + i * dcs, vdc);
+      if constexpr (GATED) {
+        if (p.dc2 != nullptr) store_stream<Tin, VEC>(dc2b, dc2o + i * dc2s, vdc2);
+      }
     }
     // Keep each step's conversions next to their use (register footprint).
     __builtin_amdgcn_sched_barrier(0);
@@ -478,12 +556,21 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
 }
 
 template <typename Tin, typename Tout>
-static bool launch_bwd(const BwdArgs& args, int vec, int steps, int threads, bool cg_in_lds, dim3 grid, size_t lds,
-                       hipStream_t stream) {
-#define QSSM_BWD_CASE(V, S, N, C)                                                                     \
-  if (vec == V && steps == S && threads == N && cg_in_lds == C) {                                     \
-    hipLaunchKernelGGL((scan_bwd_kernel<Tin, Tout, V, S, N, C>), grid, dim3(N), lds, stream, args);    \
-    return true;                                                                                      \
+static bool launch_bwd(const BwdArgs& args, int vec, int steps, int threads, bool cg_in_lds, bool gated, dim3 grid,
+                       size_t lds, hipStream_t stream) {
+  if (gated) {
+    if constexpr (sizeof(Tin) == 2 && sizeof(Tout) == 2) {
+      if (vec == 4 && steps == 8 && threads == 256 && cg_in_lds) {
+        hipLaunchKernelGGL((scan_bwd_kernel<Tin, Tout, 4, 8, 256, true, true>), grid, dim3(256), lds, stream, args);
+        return true;
+      }
+    }
+    return false;
+  }
+#define QSSM_BWD_CASE(V, S, N, C)                                                                            \
+  if (vec == V && steps == S && threads == N && cg_in_lds == C) {                                            \
+    hipLaunchKernelGGL((scan_bwd_kernel<Tin, Tout, V, S, N, C, false>), grid, dim3(N), lds, stream, args);    \
+    return true;                                                                                             \
   }
   if constexpr (sizeof(Tin) == 2 && sizeof(Tout) == 2) {
     QSSM_BWD_CASE(4, 8, 256, true)

@@ -252,6 +252,20 @@ __device__ __forceinline__ void lds_put(float* p, const float* in) {
   *reinterpret_cast<Pack<float, V>*>(p) = v;
 }
 
+// Gate activations of the SSM layer (quick_ssm/layers.py:76-82), shared by the gate prologue and the gated scans
+// so that both routes round the same values: the hardware's exp2 and reciprocal (1 ulp each), fp32 throughout.
+__device__ __forceinline__ float sigmoid_f(float z) { return __builtin_amdgcn_rcpf(1.0f + __expf(-z)); }
+
+// The value `f` has after being stored as T and read back (the rounding the layer applies when it casts the
+// scan's operands to its compute dtype, and the scan when it stores a gradient).
+template <typename T, int V>
+__device__ __forceinline__ void round_through(float* f) {
+  Words<T, V> w;
+  ElemBits<T>::template set<V>(w, f);
+#pragma unroll
+  for (int v = 0; v < V; ++v) f[v] = elem(w, v);
+}
+
 // Makes the compiler forget what it knows about a loaded operand, so that the later sweeps
 // convert it to fp32 again instead of keeping an fp32 copy of every operand alive across the
 // barriers (which would double the register footprint of a tile).
@@ -416,6 +430,10 @@ struct FwdArgs {
   const float* h_init;  // [B, D] state before the first step (null: zero)
   float* h_final;       // [B, D] state after the last step (null: not wanted)
   int64_t x_sb, x_sl, a_sb, a_sl, b_sb, b_sl, c_sb, c_sl, y_sb, y_sl, h_sb, h_sl;
+  // Gated launches: a, b, x, c point at the projection outputs A_pre, D_pre, B_in, Ca and c2 at Cb; the kernel
+  // forms a = sigmoid(A_pre), b = sigmoid(D_pre), c = silu(Ca) * Cb itself.
+  const void* c2;
+  int64_t c2_sb, c2_sl;
 };
 
 struct BwdArgs {
@@ -429,6 +447,11 @@ struct BwdArgs {
   void *dx, *da, *db, *dc;
   int64_t x_sb, x_sl, a_sb, a_sl, b_sb, b_sl, c_sb, c_sl, dy_sb, dy_sl, h_sb, h_sl;
   int64_t dx_sb, dx_sl, da_sb, da_sl, db_sb, db_sl, dc_sb, dc_sl;
+  // Gated launches: operands as in FwdArgs; dx, da, db, dc receive dB_in, dA_pre, dD_pre, dCa and dc2 dCb.
+  const void* c2;
+  int64_t c2_sb, c2_sl;
+  void* dc2;
+  int64_t dc2_sb, dc2_sl;
 };
 
 // Dynamic LDS a launch needs: per-lane maps plus the cluster's neighbour maps and one row of state.
@@ -441,12 +464,12 @@ inline size_t bwd_lds_bytes(int nth, int vec, int cols, int cluster) {
 
 // Host-side launch tables, one entry per (in dtype, out dtype) pair the library instantiates.
 // Return false if (vec, steps, threads) is not an instantiated combination.
-typedef bool (*fwd_launch_fn)(const FwdArgs&, int vec, int steps, int threads, bool c_in_lds, dim3 grid, size_t lds,
-                              hipStream_t stream);
+typedef bool (*fwd_launch_fn)(const FwdArgs&, int vec, int steps, int threads, bool c_in_lds, bool gated, dim3 grid,
+                              size_t lds, hipStream_t stream);
 // Extra dynamic LDS of the forward kernel that keeps c in LDS: 8 or 16 bytes per lane and step.
 inline size_t fwd_c_lds_bytes(int nth, int steps, int lane_bytes) { return (size_t)nth * steps * lane_bytes; }
-typedef bool (*bwd_launch_fn)(const BwdArgs&, int vec, int steps, int threads, bool cg_in_lds, dim3 grid, size_t lds,
-                              hipStream_t stream);
+typedef bool (*bwd_launch_fn)(const BwdArgs&, int vec, int steps, int threads, bool cg_in_lds, bool gated, dim3 grid,
+                              size_t lds, hipStream_t stream);
 // Extra dynamic LDS of the backward kernel that keeps c and dy in LDS.
 inline size_t bwd_cg_lds_bytes(int nth, int steps) { return (size_t)2 * nth * steps * 8; }
 

@@ -19,8 +19,15 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // (no destination registers) and read from there step by step: 16 VGPRs fewer across the
 // tile's whole life, which is one more resident workgroup per SIMD.  Needs 64 or 32 lanes per row and
 // 8 bytes per lane, so that one wavefront-wide 16-byte-per-lane load covers whole rows of the strip.
-template <typename Tin, typename Tout, int VEC, int T, int NTH, bool CLDS>
+//
+// GATED: the operands are the SSM layer's projection outputs (quick_ssm/layers.py:76-88) and the gate activations
+// happen here instead of in a pass of their own: a = sigmoid(A_pre) and b = sigmoid(D_pre) replace their
+// pre-activations in the registers that hold them (rounded to the storage type, as the layer's cast to its
+// compute dtype rounds them), c = silu(Ca) * Cb is formed step by step in the last sweep from two LDS-resident
+// operands.  The a, x, b, c tensors of the layer never exist in HBM.
+template <typename Tin, typename Tout, int VEC, int T, int NTH, bool CLDS, bool GATED>
 __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
+  static_assert(!GATED || (CLDS && sizeof(Tin) * VEC == 8), "gated scan: 16-bit projections, Ca and Cb through LDS");
   static_assert(!CLDS || ((sizeof(Tin) * VEC == 8 || sizeof(Tin) * VEC == 16) && T % 2 == 0),
                 "LDS-resident c: 8 or 16 bytes per lane, even step count");
   // 16 bytes per lane: the load that deposits c in LDS gives every lane exactly its own columns of one step.
@@ -41,6 +48,7 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   float* sH = sPX + (R - 1) * cols;      // [cols] state entering the tile
   int* sSeg = reinterpret_cast<int*>(sH + cols);
   char* sC = reinterpret_cast<char*>(sSeg) + 16;  // CLDS: [NTH / 64 waves][T rows][CROW bytes] of c
+  char* sC2 = sC + (NTH / 64) * (T * CROW);       // GATED: the same of Cb (sC then holds Ca)
 
   const int tid = threadIdx.x;
   // Workgroups go to the eight XCDs in turn, so workgroup i runs on XCD i mod 8.  Chains are dealt out so that each
@@ -106,6 +114,8 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   const uint32_t ao = (uint32_t)((j * T * (int)p.a_sl + dl) * (int)sizeof(Tin)), as = (uint32_t)p.a_sl * sizeof(Tin);
   const uint32_t bo = (uint32_t)((j * T * (int)p.b_sl + dl) * (int)sizeof(Tin)), bs = (uint32_t)p.b_sl * sizeof(Tin);
   const uint32_t co = (uint32_t)((j * T * (int)p.c_sl + dl) * (int)sizeof(Tin)), cs = (uint32_t)p.c_sl * sizeof(Tin);
+  const char* c2b = GATED ? (const char*)p.c2 + ((int64_t)bi * p.c2_sb + (int64_t)t_tile * p.c2_sl + col0) * (int64_t)sizeof(Tin) : nullptr;
+  const uint32_t c2o = GATED ? (uint32_t)((j * T * (int)p.c2_sl + dl) * (int)sizeof(Tin)) : 0u, c2s = GATED ? (uint32_t)p.c2_sl * sizeof(Tin) : 0u;
   const bool want_y = p.y != nullptr;
   const bool has_c = want_y && p.c != nullptr;
 
@@ -151,6 +161,13 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
 #pragma unroll
       for (int k = 0; k < T / 2; ++k)
         __builtin_amdgcn_global_load_lds((global_ptr_t)(src + (uint32_t)(2 * k) * cs), (lds_ptr_t)(dst + k * 1024), 16, 0, 2);
+      if constexpr (GATED) {
+        const char* src2 = c2b + (uint32_t)(j * T + half) * c2s + (uint32_t)piece * 16u;
+        char* dst2 = sC2 + (tid >> 6) * (T * 512);
+#pragma unroll
+        for (int k = 0; k < T / 2; ++k)
+          __builtin_amdgcn_global_load_lds((global_ptr_t)(src2 + (uint32_t)(2 * k) * c2s), (lds_ptr_t)(dst2 + k * 1024), 16, 0, 2);
+      }
     } else if (has_c) {
 #pragma unroll
       for (int i = 0; i < T; ++i) rc[i] = load_stream<Tin, VEC>(cb, co + i * cs);
@@ -182,6 +199,11 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
         Words<Tin, VEC> cw = fill_words<Tin, VEC>(false);
         if (dok && t0 + i < g.L) cw = load_stream<Tin, VEC>(cb, co + i * cs);
         *reinterpret_cast<Words<Tin, VEC>*>(dst + lds_row(i)) = cw;
+        if constexpr (GATED) {
+          Words<Tin, VEC> cw2 = fill_words<Tin, VEC>(false);
+          if (dok && t0 + i < g.L) cw2 = load_stream<Tin, VEC>(c2b, c2o + i * c2s);
+          *reinterpret_cast<Words<Tin, VEC>*>(dst + (sC2 - sC) + lds_row(i)) = cw2;
+        }
       }
     }
   }
@@ -224,6 +246,16 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   for (int v = 0; v < VEC; ++v) { A[v] = 1.0f; X[v] = 0.0f; }
 #pragma unroll
   for (int i = 0; i < T; ++i) {
+    if constexpr (GATED) {
+      // Steps past L and columns past D hold the identity (a = 1, b = 0) already and keep it.
+      if (tile_full || (dok && t0 + i < g.L)) {
+        float ga[VEC], gb[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) { ga[v] = sigmoid_f(elem(ra[i], v)); gb[v] = sigmoid_f(elem(rb[i], v)); }
+        ElemBits<Tin>::template set<VEC>(ra[i], ga);
+        ElemBits<Tin>::template set<VEC>(rb[i], gb);
+      }
+    }
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
       const float av = elem(ra[i], v);
@@ -358,6 +390,13 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
     Words<Tin, VEC> cw;
     if (CLDS) cw = *reinterpret_cast<const Words<Tin, VEC>*>(sC + (tid >> 6) * (T * CROW) + lds_row(i) + lds_lane);
     else cw = rc[i];
+    if constexpr (GATED) {
+      const Words<Tin, VEC> cw2 = *reinterpret_cast<const Words<Tin, VEC>*>(sC2 + (tid >> 6) * (T * CROW) + lds_row(i) + lds_lane);
+      float gc[VEC];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) { const float ca = elem(cw, v); gc[v] = ca * sigmoid_f(ca) * elem(cw2, v); }
+      ElemBits<Tin>::template set<VEC>(cw, gc);
+    }
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
       h[v] = elem(ra[i], v) * h[v] + elem(rb[i], v) * elem(rx[i], v);
@@ -381,12 +420,21 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
 }
 
 template <typename Tin, typename Tout>
-static bool launch_fwd(const FwdArgs& args, int vec, int steps, int threads, bool c_in_lds, dim3 grid, size_t lds,
-                       hipStream_t stream) {
-#define QSSM_FWD_CASE(V, S, N, C)                                                                     \
-  if (vec == V && steps == S && threads == N && c_in_lds == C) {                                      \
-    hipLaunchKernelGGL((scan_fwd_kernel<Tin, Tout, V, S, N, C>), grid, dim3(N), lds, stream, args);    \
-    return true;                                                                                      \
+static bool launch_fwd(const FwdArgs& args, int vec, int steps, int threads, bool c_in_lds, bool gated, dim3 grid,
+                       size_t lds, hipStream_t stream) {
+  if (gated) {
+    if constexpr (sizeof(Tin) == 2) {
+      if (vec == 4 && steps == 8 && threads == 256 && c_in_lds) {
+        hipLaunchKernelGGL((scan_fwd_kernel<Tin, Tout, 4, 8, 256, true, true>), grid, dim3(256), lds, stream, args);
+        return true;
+      }
+    }
+    return false;
+  }
+#define QSSM_FWD_CASE(V, S, N, C)                                                                            \
+  if (vec == V && steps == S && threads == N && c_in_lds == C) {                                             \
+    hipLaunchKernelGGL((scan_fwd_kernel<Tin, Tout, V, S, N, C, false>), grid, dim3(N), lds, stream, args);    \
+    return true;                                                                                             \
   }
   if constexpr (sizeof(Tin) == 2) {
     QSSM_FWD_CASE(4, 8, 256, true)

@@ -2,7 +2,9 @@
 
 Same constructor arguments, parameter names (so state dicts interchange) and forward keywords as
 the reference's quick_ssm/layers.py:9-107.  The projections stay on torch GEMMs; the gate
-activations and casts between them and the scan are one fused HIP pass (quick_ssm_amd/gates.py),
+activations and casts between them and the scan happen inside the scan's own launches when the
+projections are stored as the 16-bit compute dtype (quick_ssm_amd/gated_scan.py) and are one fused HIP
+pass otherwise (quick_ssm_amd/gates.py),
 the pre-norm is one fused HIP pass each way (quick_ssm_amd/norm.py), and the scan is the HIP path.  Roles of the projections
 (quick_ssm/test_swiglu_equiv.py:60-70): A_proj -> forget gate a, B_proj -> the scan's input x,
 D_proj -> input gate b, C_proj_a/C_proj_b -> SwiGLU output gate c, out_proj -> output.
@@ -14,6 +16,8 @@ from typing import Optional
 import torch
 import torch.nn as nn
 
+from . import gated_scan as _gated
+from . import scan_interface as _scan_interface
 from .gates import gate_prologue
 from .norm import rms_norm
 from .scan_interface import scan
@@ -83,12 +87,23 @@ class SSM(nn.Module):
     ) -> torch.Tensor:
         skip = x if self.use_residual else 0
         u = self.pre_norm(x) if self.use_norm else x
-        drive, forget, in_gate, out_gate = self.gates(u)
         w_dtype = self.out_proj.weight.dtype
+        out_dtype = w_dtype if scan_out_dtype is None else scan_out_dtype
+        if backend in ("auto", "hip", "triton") and u.is_cuda and not _scan_interface._HONOR_TILES:
+            # 16-bit projections stored as the compute dtype: the activations happen inside the scan's launches
+            pre = (self.A_proj(u), self.B_proj(u), self.C_proj_a(u), self.C_proj_b(u), self.D_proj(u))
+            if _gated.supported(pre, self.compute_dtype, out_dtype, checkpoint):
+                y = _gated.gated_scan(*pre, out_dtype=out_dtype)
+            else:
+                forget, drive, out_gate, in_gate = gate_prologue(*pre, self.compute_dtype)
+                y = scan(x=drive, a=forget, b=in_gate, c=out_gate, block_l=block_l, checkpoint=checkpoint,
+                         tile_b=tile_b, tile_d=tile_d, out_dtype=out_dtype, backend=backend)
+            return self.out_proj(y.to(w_dtype)) + skip
+        drive, forget, in_gate, out_gate = self.gates(u)
         y = scan(
             x=drive, a=forget, b=in_gate, c=out_gate,
             block_l=block_l, checkpoint=checkpoint, tile_b=tile_b, tile_d=tile_d,
-            out_dtype=w_dtype if scan_out_dtype is None else scan_out_dtype,
+            out_dtype=out_dtype,
             backend=backend,
         )
         return self.out_proj(y.to(w_dtype)) + skip

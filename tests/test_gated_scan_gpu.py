@@ -1,0 +1,160 @@
+"""GPU parity of the gated scan (qssm_scan_gated_forward / _backward through the C ABI): projection outputs in,
+y and the projections' gradients out, with the gate activations inside the scan's launches.
+
+Oracle: gates_oracle (float64) -> the operands rounded to the storage type where the layer rounds them
+(quick_ssm/layers.py:85-88) -> scan oracle (float64) -> scan gradients -> gates_oracle backward.  Both oracles are
+pinned in tests/test_oracle.py.  Tolerance: 1e-2 of each tensor's largest magnitude (16-bit storage).
+"""
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import TOL, assert_close
+from oracle import gates_oracle
+from quick_ssm_amd import gated_scan, hip_scan
+from quick_ssm_amd.gates import gate_prologue
+from quick_ssm_amd.scan_interface import scan
+
+pytestmark = pytest.mark.gpu
+
+NAMES = ("dA_pre", "dB_in", "dCa", "dCb", "dD_pre")
+
+
+def _projections(shape, dtype, seed):
+    """Pre-activations with the spread a trained layer shows: forget gate around sigmoid^-1(0.9 .. 0.99)."""
+    gen = torch.Generator().manual_seed(seed)
+    A_pre = torch.randn(shape, generator=gen) * 0.8 + 3.0
+    B_in = torch.randn(shape, generator=gen)
+    Ca = torch.randn(shape, generator=gen) * 1.5
+    Cb = torch.randn(shape, generator=gen)
+    D_pre = torch.randn(shape, generator=gen) * 1.5 - 1.0
+    return [t.to(dtype) for t in (A_pre, B_in, Ca, Cb, D_pre)]
+
+
+def _oracle(pre, dy, dtype):
+    A_pre, B_in, Ca, Cb, D_pre = pre
+    a, x, c, b = gates_oracle.gates_forward_f64(A_pre, B_in, Ca, Cb, D_pre)
+    ops = [torch.from_numpy(t).to(dtype) for t in (x, a, b, c)]          # as the layer stores them
+    _, y = oracle.forward_f64(*ops)
+    dx, da, db, dc = oracle.backward_f64(*ops, dy)
+    grads = gates_oracle.gates_backward_f64(da, dx, dc, db, A_pre, Ca, Cb, D_pre)
+    return y, grads
+
+
+def _run(pre, dy, gpu, out_dtype, place=lambda t, dev: t.to(dev)):
+    leaves = [place(t, gpu).detach().requires_grad_(True) for t in pre]
+    assert gated_scan.supported(leaves, pre[0].dtype, out_dtype)
+    y = gated_scan.gated_scan(*leaves, out_dtype=out_dtype)
+    y.backward(place(dy, gpu))
+    assert hip_scan.workspace_status() == 0
+    return y.detach().cpu(), [t.grad.cpu() for t in leaves]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+@pytest.mark.parametrize("shape", [(2, 700, 512), (2, 1100, 264), (1, 97, 256), (3, 33, 128), (1, 2100, 136)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_gated_scan_matches_oracle_composition(gpu, dtype, shape):
+    # whole and ragged tiles, a partial last strip, several clusters per chain, rows of 64 and of 32 lanes
+    pre = _projections(shape, dtype, seed=sum(shape))
+    dy = torch.randn(shape, generator=torch.Generator().manual_seed(7)).to(dtype)
+    y_ref, g_ref = _oracle(pre, dy, dtype)
+    y, grads = _run(pre, dy, gpu, dtype)
+    assert_close("y", y, y_ref, TOL[dtype])
+    for name, got, want in zip(NAMES, grads, g_ref):
+        assert got.dtype == dtype
+        assert_close(name, got, want, TOL[dtype])
+
+
+def test_gated_scan_with_fp32_y_takes_the_two_pass_backward(gpu):
+    # y stored as fp32 (the layer's scan_out_dtype): forward fused, backward through the prologue and the plain scan
+    shape, dtype = (2, 600, 256), torch.float16
+    pre = _projections(shape, dtype, seed=21)
+    dy = torch.randn(shape, generator=torch.Generator().manual_seed(8))
+    y_ref, g_ref = _oracle(pre, dy, dtype)
+    y, grads = _run(pre, dy, gpu, torch.float32)
+    assert y.dtype == torch.float32
+    # the operands themselves are computed here and rounded to fp16: a gate within an fp32 ulp of a tie rounds the
+    # other way than the float64 oracle's, so y carries fp16-sized differences however it is stored
+    assert_close("y", y, y_ref, 1e-3)
+    for name, got, want in zip(NAMES, grads, g_ref):
+        assert_close(name, got, want, TOL[dtype])
+
+
+def test_gated_scan_equals_prologue_plus_scan(gpu):
+    # the same values through the two-pass route: y bit for bit (same activations, same roundings, same recurrence
+    # geometry is not guaranteed, so to fp32 rounding of the carries), gradients to the rounding of a(1 - a)
+    shape, dtype = (2, 900, 384), torch.bfloat16
+    pre = _projections(shape, dtype, seed=3)
+    dy = torch.randn(shape, generator=torch.Generator().manual_seed(9)).to(dtype)
+    y, grads = _run(pre, dy, gpu, dtype)
+    leaves = [t.to(gpu).requires_grad_(True) for t in pre]
+    a, x, c, b = gate_prologue(*leaves, dtype)
+    y2 = scan(x, a, b, c)
+    y2.backward(dy.to(gpu))
+    assert_close("y", y, y2.detach().cpu().double().numpy(), 1e-2)
+    frac_equal = (y == y2.detach().cpu()).float().mean().item()
+    assert frac_equal > 0.99, frac_equal
+    for name, got, leaf in zip(NAMES, grads, leaves):
+        assert_close(name, got, leaf.grad.cpu().double().numpy(), 1e-2)
+
+
+def test_gated_scan_on_column_slices_of_one_wide_tensor(gpu):
+    # the five projections as slices of one [B, L, 5 S] GEMM output (time stride 5 S), gradients into one wide tensor
+    B, L, S, dtype = 2, 300, 256, torch.bfloat16
+    pre = _projections((B, L, S), dtype, seed=11)
+    dy = torch.randn((B, L, S), generator=torch.Generator().manual_seed(10)).to(dtype)
+    y_ref, g_ref = _oracle(pre, dy, dtype)
+    wide = torch.cat(pre, dim=-1).to(gpu).requires_grad_(True)
+    parts = [wide[..., k * S:(k + 1) * S] for k in range(5)]
+    assert gated_scan.supported(parts, dtype, dtype)
+    y = gated_scan.gated_scan(*parts)
+    y.backward(dy.to(gpu))
+    assert hip_scan.workspace_status() == 0
+    assert_close("y", y.detach().cpu(), y_ref, TOL[dtype])
+    for k, (name, want) in enumerate(zip(NAMES, g_ref)):
+        assert_close(name, wide.grad[..., k * S:(k + 1) * S].cpu(), want, TOL[dtype])
+
+
+def test_what_the_gated_launches_do_not_take(gpu):
+    pre = [t.to(gpu) for t in _projections((2, 64, 256), torch.bfloat16, seed=1)]
+    assert gated_scan.supported(pre, torch.bfloat16, torch.bfloat16)
+    assert not gated_scan.supported(pre, torch.float16, torch.float16)              # compute dtype differs from storage
+    assert not gated_scan.supported(pre, torch.bfloat16, torch.bfloat16, checkpoint=False)
+    assert not gated_scan.supported([t.float() for t in pre], torch.float32, torch.float32)
+    assert not gated_scan.supported([t[..., :100] for t in pre], torch.bfloat16, torch.bfloat16)     # S < 128
+    assert not gated_scan.supported([t[..., 4:] for t in pre], torch.bfloat16, torch.bfloat16)       # rows off 16 bytes
+    assert not gated_scan.supported([t.cpu() for t in pre], torch.bfloat16, torch.bfloat16)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_ssm_layer_with_16_bit_parameters_uses_the_gated_scan_and_matches_the_sequential_path(gpu, dtype, monkeypatch):
+    from quick_ssm_amd.layers import SSM
+
+    torch.manual_seed(0)
+    layer = SSM(hidden_size=64, state_size_mult=4.0, compute_dtype=dtype, dtype=dtype)
+    xin = torch.randn(2, 192, 64).to(dtype)
+    gout = torch.randn(2, 192, 64).to(dtype)
+    calls = []
+    real = gated_scan.gated_scan
+    monkeypatch.setattr(gated_scan, "gated_scan", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+
+    def run(mod, inp, backend):
+        mod.zero_grad(set_to_none=True)
+        inp = inp.clone().requires_grad_(True)
+        out = mod(inp, backend=backend)
+        out.backward(gout.to(inp.device))
+        return out.detach().cpu().float(), inp.grad.cpu().float(), {n: p.grad.cpu().float() for n, p in mod.named_parameters()}
+
+    ref_layer = SSM(hidden_size=64, state_size_mult=4.0, compute_dtype=dtype, dtype=dtype)
+    ref_layer.load_state_dict(layer.state_dict())
+    y_ref, dx_ref, g_ref = run(ref_layer, xin, "torch")
+    y, dx, g = run(layer.to(gpu), xin.to(gpu), "auto")
+    assert calls, "the layer did not take the gated launches"
+    tol = 2e-2 if dtype == torch.float16 else 4e-2      # 16-bit GEMMs and 16-bit parameters on both sides
+    assert_close("layer out", y, y_ref.double().numpy(), tol)
+    assert_close("layer dx", dx, dx_ref.double().numpy(), tol)
+    for n in g_ref:
+        assert_close(f"grad {n}", g[n], g_ref[n].double().numpy(), tol)
