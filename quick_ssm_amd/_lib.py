@@ -206,6 +206,34 @@ def load() -> ctypes.CDLL:
     return _lib
 
 
+class launch_stream:
+    """`with launch_stream(device) as stream:` makes `device` current if it is not already (the common case costs
+    two cheap calls instead of a device context and a Stream object) and yields the raw handle of its current
+    stream, which is what the library's entry points take."""
+
+    __slots__ = ("device", "guard")
+
+    def __init__(self, device):
+        self.device = device
+        self.guard = None
+
+    def __enter__(self) -> int:
+        import torch
+
+        index = self.device.index
+        if index is None:
+            index = torch.cuda.current_device()
+        elif index != torch.cuda.current_device():
+            self.guard = torch.cuda.device(self.device)
+            self.guard.__enter__()
+        return torch._C._cuda_getCurrentRawStream(index)
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            self.guard.__exit__(*exc)
+        return False
+
+
 def check(code: int) -> None:
     """Raise QssmError for a nonzero return code of a library call."""
     if code != 0:

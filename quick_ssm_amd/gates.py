@@ -52,8 +52,7 @@ class _GatePrologue(torch.autograd.Function):
         ins = [_rows(t, S) for t in (A_pre, B_in, Ca, Cb, D_pre)]
         rows = ins[0].shape[0]
         outs = [torch.empty((rows, S), dtype=compute_dtype, device=A_pre.device) for _ in range(4)]
-        with torch.cuda.device(A_pre.device):
-            stream = torch.cuda.current_stream(A_pre.device).cuda_stream
+        with _lib.launch_stream(A_pre.device) as stream:
             args = []
             for t in ins:
                 args += [t.data_ptr(), t.stride(0) if rows > 1 else S]
@@ -77,8 +76,7 @@ class _GatePrologue(torch.autograd.Function):
 
         gs = [dense(g) for g in (g_a, g_x, g_c, g_b)]
         outs = [torch.empty((rows, S), dtype=ctx.in_dtype, device=dev) for _ in range(5)]
-        with torch.cuda.device(dev):
-            stream = torch.cuda.current_stream(dev).cuda_stream
+        with _lib.launch_stream(dev) as stream:
             args = [g.data_ptr() for g in gs]
             for t in (A_pre, Ca, Cb, D_pre):
                 args += [t.data_ptr(), t.stride(0) if rows > 1 else S]

@@ -44,8 +44,7 @@ class _RmsNorm(torch.autograd.Function):
         w = weight.contiguous()
         y = torch.empty((rows, H), dtype=x.dtype, device=x.device)
         rstd = torch.empty((rows,), dtype=torch.float32, device=x.device)
-        with torch.cuda.device(x.device):
-            stream = torch.cuda.current_stream(x.device).cuda_stream
+        with _lib.launch_stream(x.device) as stream:
             _lib.check(_lib.load().qssm_rmsnorm_forward(
                 x2.data_ptr(), _ld(x2, H), w.data_ptr(), y.data_ptr(), rstd.data_ptr(), rows, H, float(eps),
                 _CODES[x.dtype], stream))
@@ -67,8 +66,7 @@ class _RmsNorm(torch.autograd.Function):
         dw = torch.empty((H,), dtype=w.dtype, device=dev)
         n_part = max(_lib.QSSM_RMSNORM_MIN_PARTIAL_ROWS, min(PARTIAL_ROWS, (rows + 7) // 8))
         partial = torch.empty((n_part, H), dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
-            stream = torch.cuda.current_stream(dev).cuda_stream
+        with _lib.launch_stream(dev) as stream:
             _lib.check(_lib.load().qssm_rmsnorm_backward(
                 g.data_ptr(), _ld(g, H), x2.data_ptr(), _ld(x2, H), w.data_ptr(), rstd.data_ptr(), dx.data_ptr(),
                 dw.data_ptr(), partial.data_ptr(), n_part, rows, H, ctx.eps, _CODES[x2.dtype], stream))
