@@ -34,9 +34,13 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // the last sweep turns the scan's gradients (rounded to the storage type, as the scan stores them) into the
 // projections' gradients dA_pre = da a (1 - a), dB_in = dx, dD_pre = db b (1 - b),
 // dCa = dc Cb s (1 + Ca (1 - s)), dCb = dc Ca s with s = sigmoid(Ca): no gradient of a, x, b, c ever exists in HBM.
-template <typename Tin, typename Tout, int VEC, int T, int NTH, bool CLDS, bool GATED>
+//
+// XLANE: rows of 16 lanes or fewer (a few columns of D), where a tile has 16 to 256 lane groups: their maps are
+// combined, in both directions, by exchanges between the lanes of a wavefront instead of two walks through LDS.
+template <typename Tin, typename Tout, int VEC, int T, int NTH, bool CLDS, bool GATED, bool XLANE>
 __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   static_assert(!GATED || CLDS, "gated scan: Ca, Cb and dy through LDS");
+  static_assert(!XLANE || (!CLDS && !GATED), "cross-lane fold: register-only operands");
   static_assert(!CLDS || (sizeof(Tin) * VEC == 8 && sizeof(Tout) * VEC == 8 && T % 2 == 0),
                 "LDS-resident c and dy: 8 bytes per lane, even step count");
   extern __shared__ __align__(16) float lds[];
@@ -349,56 +353,143 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
       Xe[v] = elem(ra[i], v) * (elem(cw, v) * elem(gw, v) + Xe[v]);
     __builtin_amdgcn_sched_barrier(0);
   }
-  lds_put<VEC>(sA + tid * VEC, A);
-  lds_put<VEC>(sXf + tid * VEC, Xf);
-  lds_put<VEC>(sXe + tid * VEC, Xe);
-#pragma unroll
-  for (int i = 0; i < T; ++i) {
-    forget(ra[i]); forget(rb[i]); forget(rx[i]);
-    if (!CLDS) { forget(rc[i]); forget(rg[i]); }
-  }
-  lds_barrier();
-
   // ---- compose: groups before this one (forward state), groups after it (reverse carry) --------
-  float Ap[VEC], Xp[VEC], As[VEC], Xs[VEC];
+  // Aq, Xq: the part of the reverse carry's map that the tile's total still has to be joined with; own: where the
+  // map that closes the total sits in LDS (see the edge group below).
+  float Ap[VEC], Xp[VEC], As[VEC], Xs[VEC], Aq[VEC], Xq[VEC];
+  const float* own;
+  if constexpr (XLANE) {
+    // Cross-lane scans, one each way: the groups of one wavefront combine their maps with log2(64 / G) exchanges
+    // between lanes, and one total per wavefront and direction goes through LDS.
+    const int wl = tid & 63, w = tid >> 6;
+    float* sAr = sA + NTH * VEC / 2;   // reverse totals of the wavefronts (the forward ones fill a quarter of sA at most)
+    float Ar[VEC];
 #pragma unroll
-  for (int v = 0; v < VEC; ++v) { Ap[v] = 1.0f; Xp[v] = 0.0f; As[v] = 1.0f; Xs[v] = 0.0f; }
-  if (!have_h) {
-#pragma unroll 4
-    for (int k = 0; k < j; ++k) {
-      float ak[VEC], xk[VEC];
-      lds_get<VEC>(sA + k * cols + dl, ak);
-      lds_get<VEC>(sXf + k * cols + dl, xk);
+    for (int v = 0; v < VEC; ++v) Ar[v] = A[v];
+    for (int off = G; off < 64; off <<= 1) {
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
-        Xp[v] = ak[v] * Xp[v] + xk[v];
-        Ap[v] = ak[v] * Ap[v];
+        const float pa = __shfl_up(A[v], off, 64), px = __shfl_up(Xf[v], off, 64);
+        const float qa = __shfl_down(Ar[v], off, 64), qx = __shfl_down(Xe[v], off, 64);
+        if (wl >= off) {        // forward: the earlier groups' map, then this one
+          Xf[v] = A[v] * px + Xf[v];
+          A[v] = A[v] * pa;
+        }
+        if (wl + off < 64) {    // reverse: the later groups' map, then this one
+          Xe[v] = Ar[v] * qx + Xe[v];
+          Ar[v] = Ar[v] * qa;
+        }
       }
     }
-  }
-#pragma unroll 4
-  for (int k = NG - 1; k > j; --k) {
-    float ak[VEC], xk[VEC];
-    lds_get<VEC>(sA + k * cols + dl, ak);
-    lds_get<VEC>(sXe + k * cols + dl, xk);
+    float Aef[VEC], Xef[VEC], Aer[VEC], Xer[VEC];   // the wavefront's groups before / after this one
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
-      Xs[v] = ak[v] * Xs[v] + xk[v];
-      As[v] = ak[v] * As[v];
+      Aef[v] = __shfl_up(A[v], G, 64);
+      Xef[v] = __shfl_up(Xf[v], G, 64);
+      Aer[v] = __shfl_down(Ar[v], G, 64);
+      Xer[v] = __shfl_down(Xe[v], G, 64);
+      if (wl < G) { Aef[v] = 1.0f; Xef[v] = 0.0f; }
+      if (wl >= 64 - G) { Aer[v] = 1.0f; Xer[v] = 0.0f; }
     }
+    own = sAr + dl;   // the first wavefront's reverse total: the edge group is its first group
+    if (wl >= 64 - G) {
+      lds_put<VEC>(sA + w * cols + dl, A);
+      lds_put<VEC>(sXf + w * cols + dl, Xf);
+    }
+    if (wl < G) {
+      lds_put<VEC>(sAr + w * cols + dl, Ar);
+      lds_put<VEC>(sXe + w * cols + dl, Xe);
+    }
+#pragma unroll
+    for (int i = 0; i < T; ++i) {
+      forget(ra[i]); forget(rb[i]); forget(rx[i]); forget(rc[i]); forget(rg[i]);
+    }
+    lds_barrier();
+    float Aw[VEC], Xw[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) { Aw[v] = 1.0f; Xw[v] = 0.0f; Aq[v] = 1.0f; Xq[v] = 0.0f; }
+    if (!have_h) {
+      for (int k = 0; k < w; ++k) {   // forward totals of the wavefronts before this one
+        float ak[VEC], xk[VEC];
+        lds_get<VEC>(sA + k * cols + dl, ak);
+        lds_get<VEC>(sXf + k * cols + dl, xk);
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          Xw[v] = ak[v] * Xw[v] + xk[v];
+          Aw[v] = ak[v] * Aw[v];
+        }
+      }
+    }
+    for (int k = (NTH >> 6) - 1; k > w; --k) {   // reverse totals of the wavefronts after this one
+      float ak[VEC], xk[VEC];
+      lds_get<VEC>(sAr + k * cols + dl, ak);
+      lds_get<VEC>(sXe + k * cols + dl, xk);
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        Xq[v] = ak[v] * Xq[v] + xk[v];
+        Aq[v] = ak[v] * Aq[v];
+      }
+    }
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      Ap[v] = Aef[v] * Aw[v];
+      Xp[v] = Aef[v] * Xw[v] + Xef[v];
+      As[v] = Aer[v] * Aq[v];
+      Xs[v] = Aer[v] * Xq[v] + Xer[v];
+    }
+  } else {
+    own = sA + tid * VEC;
+    lds_put<VEC>(sA + tid * VEC, A);
+    lds_put<VEC>(sXf + tid * VEC, Xf);
+    lds_put<VEC>(sXe + tid * VEC, Xe);
+#pragma unroll
+    for (int i = 0; i < T; ++i) {
+      forget(ra[i]); forget(rb[i]); forget(rx[i]);
+      if (!CLDS) { forget(rc[i]); forget(rg[i]); }
+    }
+    lds_barrier();
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) { Ap[v] = 1.0f; Xp[v] = 0.0f; As[v] = 1.0f; Xs[v] = 0.0f; }
+    if (!have_h) {
+#pragma unroll 4
+      for (int k = 0; k < j; ++k) {
+        float ak[VEC], xk[VEC];
+        lds_get<VEC>(sA + k * cols + dl, ak);
+        lds_get<VEC>(sXf + k * cols + dl, xk);
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          Xp[v] = ak[v] * Xp[v] + xk[v];
+          Ap[v] = ak[v] * Ap[v];
+        }
+      }
+    }
+#pragma unroll 4
+    for (int k = NG - 1; k > j; --k) {
+      float ak[VEC], xk[VEC];
+      lds_get<VEC>(sA + k * cols + dl, ak);
+      lds_get<VEC>(sXe + k * cols + dl, xk);
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        Xs[v] = ak[v] * Xs[v] + xk[v];
+        As[v] = ak[v] * As[v];
+      }
+    }
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) { Aq[v] = As[v]; Xq[v] = Xs[v]; }
   }
 
   // ---- reverse carry entering the tile -----------------------------------------------------------
   if (multi) {
     float At[VEC], Xt[VEC];
     if (edge) {
+      // the map that closes the tile's total (this group's own, or its wavefront's) after everything after it
       float av[VEC], xv[VEC];
-      lds_get<VEC>(sA + tid * VEC, av);
-      lds_get<VEC>(sXe + tid * VEC, xv);
+      lds_get<VEC>(own, av);
+      lds_get<VEC>(XLANE ? sXe + dl : sXe + tid * VEC, xv);
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
-        At[v] = av[v] * As[v];
-        Xt[v] = av[v] * Xs[v] + xv[v];
+        At[v] = av[v] * Aq[v];
+        Xt[v] = av[v] * Xq[v] + xv[v];
       }
       // Earlier tiles of the cluster need this tile's map; it depends on nothing, so it goes out first.
       if (dok && m > 0) {
@@ -561,16 +652,30 @@ static bool launch_bwd(const BwdArgs& args, int vec, int steps, int threads, boo
   if (gated) {
     if constexpr (sizeof(Tin) == 2 && sizeof(Tout) == 2) {
       if (vec == 4 && steps == 8 && threads == 256 && cg_in_lds) {
-        hipLaunchKernelGGL((scan_bwd_kernel<Tin, Tout, 4, 8, 256, true, true>), grid, dim3(256), lds, stream, args);
+        hipLaunchKernelGGL((scan_bwd_kernel<Tin, Tout, 4, 8, 256, true, true, false>), grid, dim3(256), lds, stream, args);
         return true;
       }
     }
     return false;
   }
-#define QSSM_BWD_CASE(V, S, N, C)                                                                            \
-  if (vec == V && steps == S && threads == N && cg_in_lds == C) {                                            \
-    hipLaunchKernelGGL((scan_bwd_kernel<Tin, Tout, V, S, N, C, false>), grid, dim3(N), lds, stream, args);    \
-    return true;                                                                                             \
+  // rows of at most 16 lanes in a 256-lane tile: 16 or more lane groups, folded across lanes
+  const bool xlane = threads == 256 && !cg_in_lds && args.g.g_log2 <= 4;
+#define QSSM_BWD_XCASE(V, S)                                                                                          \
+  if (xlane && vec == V && steps == S) {                                                                              \
+    hipLaunchKernelGGL((scan_bwd_kernel<Tin, Tout, V, S, 256, false, false, true>), grid, dim3(256), lds, stream, args); \
+    return true;                                                                                                      \
+  }
+  QSSM_BWD_XCASE(1, 4)
+  QSSM_BWD_XCASE(1, 8)
+  QSSM_BWD_XCASE(2, 4)
+  QSSM_BWD_XCASE(2, 8)
+  QSSM_BWD_XCASE(4, 4)
+  QSSM_BWD_XCASE(4, 8)
+#undef QSSM_BWD_XCASE
+#define QSSM_BWD_CASE(V, S, N, C)                                                                                   \
+  if (vec == V && steps == S && threads == N && cg_in_lds == C) {                                                   \
+    hipLaunchKernelGGL((scan_bwd_kernel<Tin, Tout, V, S, N, C, false, false>), grid, dim3(N), lds, stream, args);    \
+    return true;                                                                                                    \
   }
   if constexpr (sizeof(Tin) == 2 && sizeof(Tout) == 2) {
     QSSM_BWD_CASE(4, 8, 256, true)

@@ -25,8 +25,12 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // pre-activations in the registers that hold them (rounded to the storage type, as the layer's cast to its
 // compute dtype rounds them), c = silu(Ca) * Cb is formed step by step in the last sweep from two LDS-resident
 // operands.  The a, x, b, c tensors of the layer never exist in HBM.
-template <typename Tin, typename Tout, int VEC, int T, int NTH, bool CLDS, bool GATED>
+//
+// XLANE: rows of 16 lanes or fewer (a few columns of D), where a tile has 16 to 256 lane groups: their maps are
+// combined by exchanges between the lanes of a wavefront instead of a walk through LDS.
+template <typename Tin, typename Tout, int VEC, int T, int NTH, bool CLDS, bool GATED, bool XLANE>
 __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
+  static_assert(!XLANE || (!CLDS && !GATED), "cross-lane fold: register-only operands");
   static_assert(!GATED || (CLDS && sizeof(Tin) * VEC == 8), "gated scan: 16-bit projections, Ca and Cb through LDS");
   static_assert(!CLDS || ((sizeof(Tin) * VEC == 8 || sizeof(Tin) * VEC == 16) && T % 2 == 0),
                 "LDS-resident c: 8 or 16 bytes per lane, even step count");
@@ -264,26 +268,82 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
     }
     __builtin_amdgcn_sched_barrier(0);
   }
-  lds_put<VEC>(sA + tid * VEC, A);
-  lds_put<VEC>(sX + tid * VEC, X);
-#pragma unroll
-  for (int i = 0; i < T; ++i) { forget(ra[i]); forget(rb[i]); forget(rx[i]); }
-  lds_barrier();
-
   // ---- compose the maps of the lane groups before this one ------------------------------------
-  float Ap[VEC], Xp[VEC];
+  // Ap, Xp: the map of the tile's steps before this lane's; Aq, Xq: the part of it that the tile's total still
+  // has to be joined with (see the edge group below); own: where the map that closes the total sits in LDS.
+  float Ap[VEC], Xp[VEC], Aq[VEC], Xq[VEC];
+  const float* own;
+  if constexpr (XLANE) {   // several lane groups share a wavefront (g_log2 < 6)
+    // Cross-lane scan: the groups of one wavefront combine their maps with log2(64 / G) exchanges between lanes
+    // (group k takes the running map of group k - 2^s), whatever their number; only one total per wavefront
+    // goes through LDS.  With one lane per row (D of a few columns) a 256-lane tile has 256 groups: 6 exchanges
+    // and 3 LDS reads instead of up to 255 dependent LDS reads.
+    const int wl = tid & 63;
+    for (int off = G; off < 64; off <<= 1) {
 #pragma unroll
-  for (int v = 0; v < VEC; ++v) { Ap[v] = 1.0f; Xp[v] = 0.0f; }
-#pragma unroll 4
-  for (int k = 0; k < j; ++k) {
-    float ak[VEC], xk[VEC];
-    lds_get<VEC>(sA + k * cols + dl, ak);
-    lds_get<VEC>(sX + k * cols + dl, xk);
+      for (int v = 0; v < VEC; ++v) {
+        const float pa = __shfl_up(A[v], off, 64), px = __shfl_up(X[v], off, 64);
+        if (wl >= off) {   // the earlier groups' map (pa, px), then this one
+          X[v] = A[v] * px + X[v];
+          A[v] = A[v] * pa;
+        }
+      }
+    }
+    float Ae[VEC], Xe[VEC];   // map of the wavefront's groups before this one
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
-      Xp[v] = ak[v] * Xp[v] + xk[v];
-      Ap[v] = ak[v] * Ap[v];
+      Ae[v] = __shfl_up(A[v], G, 64);
+      Xe[v] = __shfl_up(X[v], G, 64);
+      if (wl < G) { Ae[v] = 1.0f; Xe[v] = 0.0f; }
     }
+    const int w = tid >> 6;
+    own = sA + w * cols + dl;
+    if (wl >= 64 - G) {   // the wavefront's last group now holds its total
+      lds_put<VEC>(sA + w * cols + dl, A);
+      lds_put<VEC>(sX + w * cols + dl, X);
+    }
+#pragma unroll
+    for (int i = 0; i < T; ++i) { forget(ra[i]); forget(rb[i]); forget(rx[i]); }
+    lds_barrier();
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) { Aq[v] = 1.0f; Xq[v] = 0.0f; }
+    for (int k = 0; k < w; ++k) {   // totals of the wavefronts before this one
+      float ak[VEC], xk[VEC];
+      lds_get<VEC>(sA + k * cols + dl, ak);
+      lds_get<VEC>(sX + k * cols + dl, xk);
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        Xq[v] = ak[v] * Xq[v] + xk[v];
+        Aq[v] = ak[v] * Aq[v];
+      }
+    }
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      Ap[v] = Ae[v] * Aq[v];
+      Xp[v] = Ae[v] * Xq[v] + Xe[v];
+    }
+  } else {
+    own = sA + tid * VEC;
+    lds_put<VEC>(sA + tid * VEC, A);
+    lds_put<VEC>(sX + tid * VEC, X);
+#pragma unroll
+    for (int i = 0; i < T; ++i) { forget(ra[i]); forget(rb[i]); forget(rx[i]); }
+    lds_barrier();
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) { Ap[v] = 1.0f; Xp[v] = 0.0f; }
+#pragma unroll 4
+    for (int k = 0; k < j; ++k) {
+      float ak[VEC], xk[VEC];
+      lds_get<VEC>(sA + k * cols + dl, ak);
+      lds_get<VEC>(sX + k * cols + dl, xk);
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        Xp[v] = ak[v] * Xp[v] + xk[v];
+        Ap[v] = ak[v] * Ap[v];
+      }
+    }
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) { Aq[v] = Ap[v]; Xq[v] = Xp[v]; }
   }
 
   // The loads that write c into LDS are tracked by the vector memory counter only; this wave is the
@@ -295,13 +355,14 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   if (multi) {
     float At[VEC], Xt[VEC];
     if (edge) {
+      // the map that closes the tile's total (this group's own, or its wavefront's) after everything before it
       float av[VEC], xv[VEC];
-      lds_get<VEC>(sA + tid * VEC, av);
-      lds_get<VEC>(sX + tid * VEC, xv);
+      lds_get<VEC>(own, av);
+      lds_get<VEC>(own + (sX - sA), xv);
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
-        At[v] = av[v] * Ap[v];
-        Xt[v] = av[v] * Xp[v] + xv[v];
+        At[v] = av[v] * Aq[v];
+        Xt[v] = av[v] * Xq[v] + xv[v];
       }
       // Later tiles of the cluster need this tile's map; it depends on nothing, so it goes out first.
       if (dok && m + 1 < R && seg + 1 < g.n_seg) {
@@ -425,16 +486,30 @@ static bool launch_fwd(const FwdArgs& args, int vec, int steps, int threads, boo
   if (gated) {
     if constexpr (sizeof(Tin) == 2) {
       if (vec == 4 && steps == 8 && threads == 256 && c_in_lds) {
-        hipLaunchKernelGGL((scan_fwd_kernel<Tin, Tout, 4, 8, 256, true, true>), grid, dim3(256), lds, stream, args);
+        hipLaunchKernelGGL((scan_fwd_kernel<Tin, Tout, 4, 8, 256, true, true, false>), grid, dim3(256), lds, stream, args);
         return true;
       }
     }
     return false;
   }
-#define QSSM_FWD_CASE(V, S, N, C)                                                                            \
-  if (vec == V && steps == S && threads == N && c_in_lds == C) {                                             \
-    hipLaunchKernelGGL((scan_fwd_kernel<Tin, Tout, V, S, N, C, false>), grid, dim3(N), lds, stream, args);    \
-    return true;                                                                                             \
+  // rows of at most 16 lanes in a 256-lane tile: 16 or more lane groups, folded across lanes
+  const bool xlane = threads == 256 && !c_in_lds && args.g.g_log2 <= 4;
+#define QSSM_FWD_XCASE(V, S)                                                                                          \
+  if (xlane && vec == V && steps == S) {                                                                              \
+    hipLaunchKernelGGL((scan_fwd_kernel<Tin, Tout, V, S, 256, false, false, true>), grid, dim3(256), lds, stream, args); \
+    return true;                                                                                                      \
+  }
+  QSSM_FWD_XCASE(1, 4)
+  QSSM_FWD_XCASE(1, 8)
+  QSSM_FWD_XCASE(2, 4)
+  QSSM_FWD_XCASE(2, 8)
+  QSSM_FWD_XCASE(4, 4)
+  QSSM_FWD_XCASE(4, 8)
+#undef QSSM_FWD_XCASE
+#define QSSM_FWD_CASE(V, S, N, C)                                                                                   \
+  if (vec == V && steps == S && threads == N && c_in_lds == C) {                                                    \
+    hipLaunchKernelGGL((scan_fwd_kernel<Tin, Tout, V, S, N, C, false, false>), grid, dim3(N), lds, stream, args);    \
+    return true;                                                                                                    \
   }
   if constexpr (sizeof(Tin) == 2) {
     QSSM_FWD_CASE(4, 8, 256, true)

@@ -856,6 +856,40 @@ def test_ssm_layer_matches_sequential_path(gpu):
         assert_close(f"grad {n}", g_gpu[n], g_ref[n].double().numpy(), 2e-2)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("D", [1, 4, 16])
+def test_narrow_rows_fold_across_lanes(gpu, D, dtype):
+    # A few columns only: rows of 1 to 4 lanes, 64 to 256 lane groups per tile, whose maps are combined by exchanges
+    # between the lanes of a wavefront (both directions in the backward).  Long enough for several tiles per chain.
+    # Every output against the oracle; the launch time is printed for the record (run with -s).
+    shape = (4, 6000, D)
+    x, a, b, c, dy = make_inputs(shape, dtype=dtype, seed=90 + D)
+    ref = oracle_all(x, a, b, c, dy)
+    ops = [t.to(gpu) for t in (x, a, b, c)]
+    g = dy.to(gpu)
+    fwd = hip_scan.make_plan(*shape, dtype, dtype, _lib.QSSM_FORWARD, 1, 0)
+    assert fwd.threads == 256 and fwd.g_log2 <= 4 and fwd.n_seg > 1
+    y, _, ckpt, stride = hip_scan.scan_forward(*ops, out_dtype=dtype)
+    grads = hip_scan.scan_backward(*ops, g, ckpt=ckpt, ckpt_stride=stride)
+    assert hip_scan.workspace_status() == 0
+    _check_all(dict(zip(("y", "dx", "da", "db", "dc"), (y,) + grads)), ref, TOL[dtype])
+    full = hip_scan.scan_forward(*ops, out_dtype=dtype, want_h=True, want_ckpt=False)[1]
+    grads_h = hip_scan.scan_backward(*ops, g, h=full)            # the backward that reads h folds one way only
+    _check_all(dict(zip(("y", "dx", "da", "db", "dc"), (y,) + grads_h)), ref, TOL[dtype])
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    ev[0].record()
+    for _ in range(20):
+        hip_scan.scan_forward(*ops, out_dtype=dtype)
+    ev[1].record()
+    for _ in range(20):
+        hip_scan.scan_backward(*ops, g, ckpt=ckpt, ckpt_stride=stride)
+    ev[2].record()
+    torch.cuda.synchronize()
+    print(f"narrow rows D={D} {dtype}: forward {ev[0].elapsed_time(ev[1]) * 50:.1f} us, backward "
+          f"{ev[1].elapsed_time(ev[2]) * 50:.1f} us per launch ({fwd.n_seg} tiles per chain, "
+          f"{fwd.threads >> fwd.g_log2} lane groups per tile)", flush=True)
+
+
 def test_calibration_copy_moves_every_byte(gpu):
     # qssm_copy_bytes is the kernel of known traffic that the HBM counters are scaled by: sizes that are not a
     # multiple of a workgroup's 16 KiB, one 16-byte piece, nothing
