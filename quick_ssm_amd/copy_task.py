@@ -72,7 +72,18 @@ def loss_fn(logits: torch.Tensor, labels: torch.Tensor) -> torch.Tensor:
 
 def train_step(model: nn.Module, opt: torch.optim.Optimizer, tokens: torch.Tensor, labels: torch.Tensor,
                max_norm: float = 1.0) -> Tuple[torch.Tensor, torch.Tensor]:
-    """One optimisation step (forward, loss, backward, gradient clipping at `max_norm`, AdamW).  Returns (loss, logits)."""
+    """One optimisation step (forward, loss, backward, gradient clipping at `max_norm`, AdamW).  Returns (loss, logits).
+
+    The step runs eagerly.  Recording it into a HIP graph is refused: the backward of its torch library calls (bias
+    and embedding gradients, the loss reduction, gradient clipping) records memset nodes, which this platform does
+    not replay reliably (a recording of the whole step drifted from the eager step after two replays, one of
+    forward + backward faulted on replay).  The scan launches on their own can be recorded
+    (`hip_scan.device_counted_launches`)."""
+    if tokens.is_cuda and torch.cuda.is_current_stream_capturing():
+        raise RuntimeError(
+            "quick_ssm_amd.copy_task.train_step cannot be recorded into a HIP graph: its torch library calls record "
+            "memset nodes that do not replay reliably on this platform. Run the step eagerly; scan launches alone "
+            "can be recorded (hip_scan.device_counted_launches).")
     logits = model(tokens)
     loss = loss_fn(logits, labels)
     opt.zero_grad(set_to_none=True)

@@ -85,6 +85,14 @@ class SSM(nn.Module):
         backend: str = "auto",
         scan_out_dtype: Optional[torch.dtype] = None,
     ) -> torch.Tensor:
+        if (x.is_cuda and torch.cuda.is_current_stream_capturing() and torch.is_grad_enabled()
+                and (x.requires_grad or any(p.requires_grad for p in self.parameters()))):
+            # a recorded training step would also record the backward of the projections' bias and weight gradients
+            # (library reductions with memset nodes), which does not replay reliably on this platform
+            raise RuntimeError(
+                "quick_ssm_amd.SSM: recording a differentiable forward into a HIP graph is not supported (the backward's "
+                "torch library calls record memset nodes that do not replay reliably on this platform); record under "
+                "torch.no_grad(), or run the training step eagerly.")
         skip = x if self.use_residual else 0
         u = self.pre_norm(x) if self.use_norm else x
         w_dtype = self.out_proj.weight.dtype

@@ -57,3 +57,32 @@ def test_training_step_on_hip_matches_sequential_path(gpu, dtype):
     # only loosely: the direction of a near-zero gradient component is rounding noise
     worst = max(float((a - b).abs().max()) for a, b in zip(p0, p1))
     assert worst <= 2.5e-3, worst
+
+
+@pytest.mark.gpu
+def test_recording_the_training_step_is_refused_before_anything_is_recorded(gpu):
+    # whole-step graph capture is unsupported (library memset nodes do not replay reliably here): the harness and the
+    # layer say so instead of recording; nothing is launched inside the refused recordings
+    import warnings
+
+    from quick_ssm_amd.layers import SSM
+
+    torch.manual_seed(0)
+    model = copy_task.CopyStack(hidden=32, layers=1, compute_dtype=torch.float32, device=gpu)
+    opt = torch.optim.AdamW(model.parameters(), lr=1e-3)
+    tokens, labels = copy_task.build_teacher_batch(2, 8, gpu, generator=torch.Generator().manual_seed(1))
+    copy_task.train_step(model, opt, tokens, labels)            # eager: fine
+    layer = SSM(32, 2.0, device=gpu)
+    xin = torch.randn(2, 16, 32, device=gpu)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side), warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        with pytest.raises(RuntimeError, match="cannot be recorded"):
+            with torch.cuda.graph(torch.cuda.CUDAGraph(), stream=side):
+                copy_task.train_step(model, opt, tokens, labels)
+        with pytest.raises(RuntimeError, match="not supported"):
+            with torch.cuda.graph(torch.cuda.CUDAGraph(), stream=side):
+                layer(xin)
+    torch.cuda.synchronize()
+    loss, _ = copy_task.train_step(model, opt, tokens, labels)  # and the eager step still works afterwards
+    assert torch.isfinite(loss)
