@@ -83,7 +83,9 @@ typedef struct qssm_plan {
   int32_t ckpt_stride;    /* spacing (time steps) of saved states; divides seg_len */
   int32_t n_ckpt;         /* ceil(L / ckpt_stride) */
   int32_t lds_bytes;      /* dynamic LDS per workgroup */
-  int32_t reserved;
+  int32_t keep_tiles;     /* forward: the last keep_tiles tiles of every chain load their operands with ordinary
+                             loads, so that the backward, which starts there, finds them in the caches; the rest
+                             streams past the caches.  0 switches it off. */
   uint64_t control_bytes;   /* control block the launch needs (status word + ticket counters) */
   uint64_t workspace_bytes; /* workspace the launch needs (words exchanged between workgroups) */
   uint64_t ckpt_elems;      /* B * n_ckpt * D floats */

@@ -69,14 +69,14 @@ class Plan(ctypes.Structure):
         ("ckpt_stride", ctypes.c_int32),
         ("n_ckpt", ctypes.c_int32),
         ("lds_bytes", ctypes.c_int32),
-        ("reserved", ctypes.c_int32),
+        ("keep_tiles", ctypes.c_int32),
         ("control_bytes", ctypes.c_uint64),
         ("workspace_bytes", ctypes.c_uint64),
         ("ckpt_elems", ctypes.c_uint64),
     ]
 
     def describe(self) -> dict:
-        return {name: int(getattr(self, name)) for name, _ in self._fields_ if name != "reserved"}
+        return {name: int(getattr(self, name)) for name, _ in self._fields_}
 
 
 class Strides(ctypes.Structure):

@@ -152,18 +152,21 @@ __device__ __forceinline__ float elem(const Words<T, V>& p, int v) {
 }
 
 // One vector load / store of VEC elements at a byte offset from a workgroup-uniform base.
-// Operands and results are touched exactly once, so they are marked non-temporal (streaming).
-template <typename T, int V>
+// Operands and results are touched exactly once by a launch, so they are marked non-temporal (streaming); KEEP
+// asks for an ordinary load instead, whose lines stay in the caches for a launch that follows.
+template <typename T, int V, bool KEEP = false>
 __device__ __forceinline__ Words<T, V> load_stream(const char* base, uint32_t byte_off) {
   if constexpr (sizeof(T) * V == 32) {   // two 16-byte halves
-    const Words<T, V / 2> lo = load_stream<T, V / 2>(base, byte_off), hi = load_stream<T, V / 2>(base, byte_off + 16u);
+    const Words<T, V / 2> lo = load_stream<T, V / 2, KEEP>(base, byte_off), hi = load_stream<T, V / 2, KEEP>(base, byte_off + 16u);
     Words<T, V> out;
 #pragma unroll
     for (int k = 0; k < 4; ++k) { out.w[k] = lo.w[k]; out.w[4 + k] = hi.w[k]; }
     return out;
   } else {
   typedef typename RawOf<sizeof(T) * V>::type raw_t;
-  const raw_t r = __builtin_nontemporal_load(reinterpret_cast<const raw_t*>(base + byte_off));
+  raw_t r;
+  if constexpr (KEEP) r = *reinterpret_cast<const raw_t*>(base + byte_off);
+  else r = __builtin_nontemporal_load(reinterpret_cast<const raw_t*>(base + byte_off));
   Words<T, V> out;
   if constexpr (sizeof(T) * V <= 4) {
     out.w[0] = (uint32_t)r;
@@ -413,6 +416,7 @@ struct Geometry {
   int n_super;      // clusters per chain
   int ckpt_stride;  // spacing of saved states
   int n_ckpt;       // saved states per (batch, column)
+  int keep_from;    // forward: tiles from this index on load their operands with ordinary (cached) loads
   unsigned epoch;   // this launch's flag value (nonzero), when the host counts launches
   const unsigned* launch_count;  // else: launches counted on the device; the flag value is *launch_count + 1
   int* status;

@@ -143,18 +143,25 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   // ---- issue every load of the tile before touching any of them ------------------------------
   Words<Tin, VEC> rx[T], ra[T], rb[T], rc[CLDS ? 1 : T];
   const bool tile_full = (t_tile + g.seg_len <= g.L) && ((strip + 1) * cols <= g.D);
-  if (tile_full) {
+  // Operand loads of a whole tile.  KEEP: ordinary loads, which leave the lines in the cache hierarchy, for the last
+  // tiles of a chain: a backward that follows the forward reads exactly those first.  Everything else streams.
+  auto load_tile = [&](auto keep_tag) {
+    constexpr bool KEEP = decltype(keep_tag)::value;
+    constexpr int AUX = KEEP ? 0 : 2;   // cache policy bits of the loads into LDS: 2 = non-temporal
+    // Loads that differ in nothing but their cache policy look alike to the optimizer, which would hoist one
+    // (ordinary) copy in front of the branch; a fence at the head of one flavour keeps them apart.
+    if constexpr (KEEP) asm volatile("" ::: "memory");
 #pragma unroll
     for (int i = 0; i < T; ++i) {
-      ra[i] = load_stream<Tin, VEC>(ab, ao + i * as);
-      rb[i] = load_stream<Tin, VEC>(bb, bo + i * bs);
-      rx[i] = load_stream<Tin, VEC>(xb, xo + i * xs);
+      ra[i] = load_stream<Tin, VEC, KEEP>(ab, ao + i * as);
+      rb[i] = load_stream<Tin, VEC, KEEP>(bb, bo + i * bs);
+      rx[i] = load_stream<Tin, VEC, KEEP>(xb, xo + i * xs);
     }
     if (CLDS && WIDE) {
       char* dst = sC + (tid >> 6) * (T * CROW);
 #pragma unroll
       for (int i = 0; i < T; ++i)
-        __builtin_amdgcn_global_load_lds((global_ptr_t)(cb + co + i * cs), (lds_ptr_t)(dst + i * 1024), 16, 0, 2);
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(cb + co + i * cs), (lds_ptr_t)(dst + i * 1024), 16, 0, AUX);
     } else if (CLDS) {
       // 16 bytes per lane: the first half of a lane group's lanes fetches one row of the strip, the second half
       // the next one (64 lanes per row: a wavefront covers two rows of one group; 32: two rows of two groups)
@@ -164,18 +171,22 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
       char* dst = sC + (tid >> 6) * (T * 512);
 #pragma unroll
       for (int k = 0; k < T / 2; ++k)
-        __builtin_amdgcn_global_load_lds((global_ptr_t)(src + (uint32_t)(2 * k) * cs), (lds_ptr_t)(dst + k * 1024), 16, 0, 2);
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(src + (uint32_t)(2 * k) * cs), (lds_ptr_t)(dst + k * 1024), 16, 0, AUX);
       if constexpr (GATED) {
         const char* src2 = c2b + (uint32_t)(j * T + half) * c2s + (uint32_t)piece * 16u;
         char* dst2 = sC2 + (tid >> 6) * (T * 512);
 #pragma unroll
         for (int k = 0; k < T / 2; ++k)
-          __builtin_amdgcn_global_load_lds((global_ptr_t)(src2 + (uint32_t)(2 * k) * c2s), (lds_ptr_t)(dst2 + k * 1024), 16, 0, 2);
+          __builtin_amdgcn_global_load_lds((global_ptr_t)(src2 + (uint32_t)(2 * k) * c2s), (lds_ptr_t)(dst2 + k * 1024), 16, 0, AUX);
       }
     } else if (has_c) {
 #pragma unroll
-      for (int i = 0; i < T; ++i) rc[i] = load_stream<Tin, VEC>(cb, co + i * cs);
+      for (int i = 0; i < T; ++i) rc[i] = load_stream<Tin, VEC, KEEP>(cb, co + i * cs);
     }
+  };
+  if (tile_full) {
+    if (seg >= g.keep_from) load_tile(std::true_type{});
+    else load_tile(std::false_type{});
   } else {
     // Steps past L and columns past D act as the identity map (a = 1, b*x = 0).
 #pragma unroll

@@ -56,9 +56,22 @@ def test_plans_are_consistent_and_forward_follows_backward(hip_lib, shape, dtype
             assert p.n_ckpt == -(-L // p.ckpt_stride)
         assert fwd.ckpt_stride == bwd.seg_len == bwd.ckpt_stride
         assert fwd.ckpt_stride % fwd.steps == 0
+        # the forward leaves the operands of its last tiles in the caches, as far as 192 MiB reach; the backward none
+        per_index = B * fwd.n_strips * fwd.strip_cols * fwd.seg_len * 4 * fwd_elem_bytes(dtype)
+        assert fwd.keep_tiles == min(fwd.n_seg, (192 << 20) // per_index) and bwd.keep_tiles == 0
         # a backward planned later, with worse alignment, still reads the same saved states
         late = hip_scan.make_plan(B, L, D, dtype, dtype, _lib.QSSM_BACKWARD, 1, bwd.seg_len)
         assert late.ckpt_stride == bwd.seg_len and late.seg_len % late.ckpt_stride == 0
+
+
+def fwd_elem_bytes(dtype):
+    return torch.empty((), dtype=dtype).element_size()
+
+
+def test_keep_tiles_of_the_headline_shape(hip_lib):
+    bf = torch.bfloat16
+    fwd = hip_scan.make_plan(8, 4096, 2048, bf, bf, _lib.QSSM_FORWARD, 8, 32)
+    assert (fwd.vec, fwd.n_seg, fwd.keep_tiles) == (8, 64, 24)
 
 
 def test_plan_rejects_bad_arguments(hip_lib):

@@ -963,3 +963,45 @@ def test_nan_in_an_input_stays_in_its_column_and_nothing_hangs(gpu):
     assert torch.isnan(y[0, 100:, 5]).all() and torch.isfinite(y[0, :100, 5]).all()
     assert torch.isfinite(got["dx"].float()).all()
     assert int(torch.isnan(got["db"].float()).sum()) == 1
+
+
+def test_tiles_that_keep_their_operands_in_the_caches_change_nothing(gpu, hip_lib):
+    # keep_tiles only chooses between streaming and ordinary loads: every setting gives the same bits
+    import ctypes
+
+    from quick_ssm_amd._lib import Plan, Strides
+
+    lib = hip_lib
+    stream = torch.cuda.current_stream(gpu).cuda_stream
+    for shape, dtype in (((2, 1100, 512), torch.bfloat16), ((2, 700, 96), torch.float32), ((1, 900, 264), torch.float16)):
+        B, L, D = shape
+        x, a, b, c, _ = make_inputs(shape, dtype=dtype, seed=5)
+        xd, ad, bd, cd = (t.to(gpu) for t in (x, a, b, c))
+        stride = hip_scan.make_plan(B, L, D, dtype, dtype, _lib.QSSM_BACKWARD, 8, 0).seg_len
+        base = hip_scan.make_plan(B, L, D, dtype, dtype, _lib.QSSM_FORWARD, 8, stride)
+        assert base.n_seg > 2
+        outs = []
+        for keep in (0, 1, base.n_seg // 2, base.n_seg, base.n_seg + 5):
+            plan = Plan.from_buffer_copy(base)
+            plan.keep_tiles = keep
+            y = torch.full(shape, float("nan"), dtype=dtype, device=gpu)
+            ck = torch.full((B, plan.n_ckpt, D), float("nan"), dtype=torch.float32, device=gpu)
+            ctl = torch.zeros(max(int(plan.control_bytes), 64), dtype=torch.uint8, device=gpu)
+            ws = torch.zeros(max(int(plan.workspace_bytes), 256), dtype=torch.uint8, device=gpu)
+            st = lambda t: Strides(t.stride(0), t.stride(1))
+            rc = lib.qssm_scan_forward(ctypes.byref(plan), xd.data_ptr(), st(xd), ad.data_ptr(), st(ad), bd.data_ptr(),
+                                       st(bd), cd.data_ptr(), st(cd), y.data_ptr(), st(y), None, Strides(0, 0),
+                                       ck.data_ptr(), ctl.data_ptr(), ctl.numel(), ws.data_ptr(), ws.numel(), 1, stream)
+            assert rc == 0, lib.qssm_error_string()
+            torch.cuda.synchronize()
+            outs.append((y, ck))
+        _, y_ref = oracle.forward_f64(x, a, b, c)
+        assert_close("y", outs[0][0].cpu(), y_ref, TOL[dtype])
+        for y, ck in outs[1:]:
+            assert torch.equal(y, outs[0][0]) and torch.equal(ck, outs[0][1])
+        plan = Plan.from_buffer_copy(base)
+        plan.keep_tiles = -1
+        rc = lib.qssm_scan_forward(ctypes.byref(plan), xd.data_ptr(), st(xd), ad.data_ptr(), st(ad), bd.data_ptr(),
+                                   st(bd), cd.data_ptr(), st(cd), y.data_ptr(), st(y), None, Strides(0, 0),
+                                   ck.data_ptr(), ctl.data_ptr(), ctl.numel(), ws.data_ptr(), ws.numel(), 1, stream)
+        assert rc == _lib.QSSM_EINVAL
