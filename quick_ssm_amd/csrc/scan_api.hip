@@ -221,9 +221,12 @@ int qssm_plan_scan_gated(int32_t B, int32_t L, int32_t D, int32_t dtype, int32_t
   int rc = qssm_plan_scan_tuned(B, L, D, dtype, out_dtype, direction, align_elems, ckpt_stride, kGatedTune, plan);
   if (rc != 0 || B == 0 || L == 0) return rc;
   int g_log2 = plan->g_log2 > 6 ? 6 : (plan->g_log2 < 5 ? 5 : plan->g_log2);
-  if (g_log2 != plan->g_log2 || plan->cluster > 2)   // same strips, more hand-overs, less LDS
+  if (g_log2 != plan->g_log2)
     rc = qssm_plan_scan_tuned(B, L, D, dtype, out_dtype, direction, align_elems, ckpt_stride,
-                              kGatedTune | (g_log2 + 1) | ((plan->cluster > 2 ? 2 : 0) << 28), plan);
+                              kGatedTune | (g_log2 + 1), plan);
+  if (rc == 0 && plan->cluster > 2)   // same strips, more hand-overs, less LDS
+    rc = qssm_plan_scan_tuned(B, L, D, dtype, out_dtype, direction, align_elems, ckpt_stride,
+                              kGatedTune | (g_log2 + 1) | (2 << 28), plan);
   if (rc != 0) return rc;
   if (plan->vec != 4 || plan->steps != 8 || plan->threads != 256 || (plan->g_log2 != 6 && plan->g_log2 != 5) ||
       plan->cluster > 2)
@@ -361,29 +364,41 @@ int qssm_plan_scan_tuned(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int3
   plan->n_seg = (L + plan->seg_len - 1) / plan->seg_len;
   plan->n_ckpt = (L + plan->ckpt_stride - 1) / plan->ckpt_stride;
 
-  // Cluster size: each cluster boundary is one serial hand-over (about 2 us under load on MI355X)
-  // that every chain pays in turn; keep their number per chain at 64 or fewer when LDS allows.
-  // Inside a cluster a tile reads the maps of all earlier tiles, and every exchanged word lengthens
-  // the tile's stay on its compute unit, so clusters stay small.
-  int cluster = 1;
-  const int tune_r = (tune >> 28) & 0xf;
-  if (tune_r >= 1) {
-    cluster = 1 << (tune_r - 1);
-  } else {
-    while (cluster < 8 && (plan->n_seg + cluster - 1) / cluster > 64) cluster <<= 1;
-    if (cluster < 2 && plan->n_seg > 8) cluster = 2;
-    // A chain of single tiles exchanges the fewest words (no maps at all, 1.9 % less traffic on the forward than
-    // clusters of two), and hands a state on in about 2.1 us.  Where a chain of that many hand-overs still ends
-    // well inside the time the launch needs to stream its operands (taken at 5.6 TB/s), it is the better trade
-    // (bf16 B=16 L=4096 D=2048 forward: 233 us against 237); where it does not (the same at B=8: 64 hand-overs in
-    // 116 us), the chain would set the pace and clusters stay.
-    const double stream_us = (double)B * L * D * (direction == QSSM_FORWARD ? 4 * es + os : 8 * es + os) / 5.6e6;
-    if (cluster > 1 && plan->n_seg * 2.1 <= 0.6 * stream_us) cluster = 1;
-  }
+  // Cluster size R.  Each cluster boundary is one serial hand-over (about 2.1 us forward, 1.8 us backward under
+  // load on MI355X) that every chain pays in turn; inside a cluster a tile reads the maps of all earlier tiles,
+  // which costs traffic and LDS (measured against R = 2 on bf16 B=8 L=4096 D=2048: +2 % at R = 4, +3.5 % forward
+  // and +10 % backward at R = 8; R = 1 has no maps at all, -2 %).  A launch takes the longer of its stream time
+  // (operands at 5.6 TB/s, with that factor) and its chain (clusters x hand-over): the R with the smaller estimate
+  // wins, the smaller R on a tie.  Large launches so get R = 1 or 2, long or narrow ones, whose chains would set
+  // the pace, up to 8 (bf16 B=2 L=8192 D=512: forward 84.5 -> 36.3 us, backward 75.6 -> 43.1 us; B=2 L=4096
+  // D=2048: 46.9 -> 36.3 and 86.2 -> 68.2 us).  Single tiles per cluster only with a wide margin (chain within
+  // 0.6 of the stream time): bf16 B=16 L=4096 D=2048 forward 233 us against 237, but at B=8 its 64 hand-overs in
+  // 116 us would set the pace.
   auto lds_for = [&](int r) -> size_t {
     return direction == QSSM_FORWARD ? fwd_lds_bytes(threads, vec, plan->strip_cols, r)
                                      : bwd_lds_bytes(threads, vec, plan->strip_cols, r);
   };
+  int cluster = 1;
+  const int tune_r = (tune >> 28) & 0xf;
+  if (tune_r >= 1) {
+    cluster = 1 << (tune_r - 1);
+  } else if (plan->n_seg > 1) {
+    static const double kMapCost[2][4] = {{-0.02, 0.0, 0.02, 0.035}, {-0.02, 0.0, 0.02, 0.10}};
+    const double hop_us = direction == QSSM_FORWARD ? 2.1 : 1.8;
+    const double stream_us = (double)B * L * D * (direction == QSSM_FORWARD ? 4 * es + os : 8 * es + os) / 5.6e6;
+    double best = 0.0;
+    cluster = 0;
+    for (int k = 0; k < 4; ++k) {
+      const int r = 1 << k;
+      if (lds_for(r) > (size_t)kMaxLdsBytes) break;
+      const double chain_us = (double)((plan->n_seg + r - 1) / r) * hop_us;
+      if (r == 1 && chain_us > 0.6 * stream_us) continue;
+      const double a = stream_us * (1.0 + kMapCost[direction == QSSM_FORWARD ? 0 : 1][k]);
+      const double est = a > chain_us ? a : chain_us;
+      if (cluster == 0 || est < best) { best = est; cluster = r; }
+    }
+    if (cluster == 0) cluster = 1;
+  }
   while (cluster > 1 && lds_for(cluster) > (size_t)kMaxLdsBytes) cluster >>= 1;
   if (lds_for(cluster) > (size_t)kMaxLdsBytes) return fail(QSSM_EINVAL, "geometry needs too much LDS");
   plan->cluster = cluster;

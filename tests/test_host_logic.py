@@ -74,6 +74,22 @@ def test_keep_tiles_of_the_headline_shape(hip_lib):
     assert (fwd.vec, fwd.n_seg, fwd.keep_tiles) == (8, 64, 24)
 
 
+def test_cluster_size_follows_stream_time_against_chain_time(hip_lib):
+    bf, f16 = torch.bfloat16, torch.float16
+
+    def clusters(B, L, D, dt, odt):
+        bwd = hip_scan.make_plan(B, L, D, dt, odt, _lib.QSSM_BACKWARD, 8, 0)
+        fwd = hip_scan.make_plan(B, L, D, dt, odt, _lib.QSSM_FORWARD, 8, bwd.seg_len)
+        return fwd.cluster, bwd.cluster
+
+    assert clusters(8, 4096, 2048, bf, bf) == (2, 2)          # chain and stream in balance
+    assert clusters(16, 4096, 2048, bf, bf) == (1, 1)         # stream time dwarfs the chain: no maps at all
+    assert clusters(1, 65536, 4096, f16, f16) == (4, 4)       # very long chains
+    assert clusters(2, 8192, 512, bf, bf) == (8, 8)           # little to stream, long chains: fewest hand-overs
+    assert clusters(2, 4096, 2048, bf, bf) == (8, 4)          # the backward pays more per neighbour map
+    assert clusters(32, 64, 1024, f16, torch.float32) == (1, 1)   # one tile per chain
+
+
 def test_plan_rejects_bad_arguments(hip_lib):
     with pytest.raises(_lib.QssmError):
         hip_scan.make_plan(-1, 4, 4, torch.float32, torch.float32, 0, 4)
