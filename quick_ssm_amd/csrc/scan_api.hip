@@ -266,8 +266,12 @@ int qssm_plan_scan_tuned(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int3
   // (a, b, x of 8 steps: 96 registers) does not leave room for the backward's rebuilt states, so the backward
   // stays at 8 bytes per lane (16 bytes at 4 steps per lane measured 240 us against 220).
   const bool wide_ok = direction == QSSM_FORWARD && es == 2 && align_elems % 8 == 0 && D % 8 == 0;
+  // It pays from about a dozen tiles per compute unit on (bf16 B=12 L=4096 D=2048: 179 us against 195; B=16
+  // L=2048 D=1024, 2048 tiles: 76 against 71), and not where few chains over a long sequence call for rows of half
+  // the width further down (fp16 B=1 L=65536 D=4096: 508 against 491 with 8 bytes per lane and 512 lanes).
+  const int64_t wide_chains = (int64_t)B * ((D + 255) / 256);
   const bool wide_auto = direction == QSSM_FORWARD && tune_vec == 0 && os == 2 && D >= 256 &&
-                         (int64_t)B * ((D + 255) / 256) * ((L + 63) / 64) >= 2 * kCUs;
+                         wide_chains * ((L + 63) / 64) >= 12 * kCUs && !(wide_chains < 32 && L >= 256 * 64);
   if (wide_ok && (tune_vec == 8 || wide_auto)) vec = 8;
   while (vec > 1 && (align_elems % vec != 0 || (D > 0 && D % vec != 0))) vec >>= 1;
   plan->vec = vec;

@@ -74,6 +74,19 @@ def test_keep_tiles_of_the_headline_shape(hip_lib):
     assert (fwd.vec, fwd.n_seg, fwd.keep_tiles) == (8, 64, 24)
 
 
+def test_sixteen_bytes_per_lane_only_where_it_pays(hip_lib):
+    bf, f16 = torch.bfloat16, torch.float16
+
+    def fwd(B, L, D, dt):
+        return hip_scan.make_plan(B, L, D, dt, dt, _lib.QSSM_FORWARD, 8, 32)
+
+    assert (fwd(8, 4096, 2048, bf).vec, fwd(12, 4096, 2048, bf).vec) == (8, 8)
+    small = fwd(16, 2048, 1024, bf)                      # 2048 tiles: too few
+    assert (small.vec, small.threads) == (4, 512)
+    long = fwd(1, 65536, 4096, f16)                      # 16 strips over a long sequence: rows of half the width instead
+    assert (long.vec, long.threads, long.g_log2) == (4, 512, 5)
+
+
 def test_cluster_size_follows_stream_time_against_chain_time(hip_lib):
     bf, f16 = torch.bfloat16, torch.float16
 
