@@ -637,7 +637,7 @@ static int backward_launch(const qssm_plan* plan, const void* x, qssm_strides sx
   // c and dy can live in LDS instead of registers when a row of the strip is one wavefront of 8-byte
   // lanes in both and their rows can be fetched 16 bytes at a time.
   size_t lds = (size_t)plan->lds_bytes;
-  bool cg_in_lds = es == 2 && os == 2 && v == 4 && (plan->g_log2 == 6 || plan->g_log2 == 5) && plan->steps == 8 && plan->threads == 256 &&
+  bool cg_in_lds = es == 2 && (os == 2 || os == 4) && v == 4 && (plan->g_log2 == 6 || plan->g_log2 == 5) && plan->steps == 8 && plan->threads == 256 &&
                    ((uintptr_t)c) % 16 == 0 && (sc.b * es) % 16 == 0 && (sc.l * es) % 16 == 0 &&
                    ((uintptr_t)dy) % 16 == 0 && (sdy.b * os) % 16 == 0 && (sdy.l * os) % 16 == 0 &&
                    lds + bwd_cg_lds_bytes(plan->threads, plan->steps) <= (size_t)kMaxLdsBytes;

@@ -26,7 +26,9 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // CLDS: c and dy are loaded straight into LDS (no destination registers) and read from there in the
 // sweeps that use them: 32 VGPRs fewer across the tile's whole life, which is one more resident
 // workgroup per SIMD.  Needs 64 lanes per row and 8 bytes per lane in both tensors, so that one
-// wavefront-wide 16-byte-per-lane load covers two rows of the strip.
+// wavefront-wide 16-byte-per-lane load covers two rows of the strip.  With 16-bit operands and fp32 dy (16 bytes
+// per lane) only dy goes through LDS, every lane fetching its own piece, and c stays in registers: LDS has room
+// for one 16-byte or two 8-byte operands at three workgroups per compute unit, and dy is the larger one.
 //
 // GATED: the operands are the SSM layer's projection outputs (quick_ssm/layers.py:76-88) and both the gate
 // activations and their derivatives happen here: a = sigmoid(A_pre), b = sigmoid(D_pre) replace their
@@ -41,8 +43,11 @@ template <typename Tin, typename Tout, int VEC, int T, int NTH, bool CLDS, bool 
 __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   static_assert(!GATED || CLDS, "gated scan: Ca, Cb and dy through LDS");
   static_assert(!XLANE || (!CLDS && !GATED), "cross-lane fold: register-only operands");
-  static_assert(!CLDS || (sizeof(Tin) * VEC == 8 && sizeof(Tout) * VEC == 8 && T % 2 == 0),
-                "LDS-resident c and dy: 8 bytes per lane, even step count");
+  static_assert(!CLDS || (sizeof(Tin) * VEC == 8 && (sizeof(Tout) * VEC == 8 || sizeof(Tout) * VEC == 16) && T % 2 == 0),
+                "LDS-resident c and dy: 8 bytes per lane (dy alone: 16), even step count");
+  static_assert(!GATED || sizeof(Tout) * VEC == 8, "gated scan: 16-bit dy");
+  constexpr bool GW = CLDS && sizeof(Tout) * VEC == 16;   // dy alone in LDS, 16 bytes per lane
+  constexpr bool CREG = !CLDS || GW;                       // c in registers
   extern __shared__ __align__(16) float lds[];
   const Geometry& g = p.g;
   const int G = 1 << g.g_log2;
@@ -59,12 +64,16 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   float* sE = sPX + (R - 1) * cols;      // [cols] reverse carry entering the tile
   int* sSeg = reinterpret_cast<int*>(sE + cols);
   char* sC = reinterpret_cast<char*>(sSeg) + 16 + ((int)threadIdx.x >> 6) * (T * 512);  // CLDS: this wave's [T rows][512 bytes] of c
-  char* sG = sC + (NTH / 64) * (T * 512);                                  // and of dy
+  // and of dy; with 16 bytes per lane dy has the block to itself: [T rows][64 lanes x 16 bytes] per wave
+  char* sG = GW ? reinterpret_cast<char*>(sSeg) + 16 + ((int)threadIdx.x >> 6) * (T * 1024) : sC + (NTH / 64) * (T * 512);
   char* sC2 = sG + (NTH / 64) * (T * 512);                                 // GATED: and of Cb (sC then holds Ca)
   // Where step i of this lane sits in its wavefront's LDS block: the loads that fill it deposit 1024 bytes per
   // instruction in lane order, i.e. per pair of steps [group in wavefront][step parity][G * 8 bytes].
   const int lds_lane = (((int)threadIdx.x & 63) >> g.g_log2) * (G * 16) + ((int)threadIdx.x & (G - 1)) * 8;
   auto lds_row = [&](int i) { return (i >> 1) * 1024 + (i & 1) * (G * 8); };
+  auto g_slot = [&](int i) -> char* {   // where dy of this lane's step i sits
+    return GW ? sG + i * 1024 + ((int)threadIdx.x & 63) * 16 : sG + lds_row(i) + lds_lane;
+  };
 
   const int tid = threadIdx.x;
   // Workgroups go to the eight XCDs in turn, so workgroup i runs on XCD i mod 8.  Chains are dealt out so that each
@@ -152,7 +161,7 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   if (want_state) pk_state.issue(next_state, G);
 
   // ---- issue every load of the tile before touching any of them ------------------------------
-  Words<Tin, VEC> rx[T], ra[T], rb[T], rc[CLDS ? 1 : T];
+  Words<Tin, VEC> rx[T], ra[T], rb[T], rc[CREG ? T : 1];
   Words<Tout, VEC> rg[CLDS ? 1 : T];
   float hs[T][VEC];   // h(t0 + i)
   float hprev[VEC];   // h(t0 - 1); before the rebuild, the state at the tile's first step
@@ -166,6 +175,13 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
         rb[i] = load_stream<Tin, VEC>(bb, bo + i * bs);
         rx[i] = load_stream<Tin, VEC>(xb, xo + i * xs);
       }
+      if constexpr (GW) {
+#pragma unroll
+        for (int i = 0; i < T; ++i) rc[i] = load_stream<Tin, VEC>(cb, co + i * cs);
+#pragma unroll
+        for (int i = 0; i < T; ++i)
+          __builtin_amdgcn_global_load_lds((global_ptr_t)(gb + go + i * gs), (lds_ptr_t)(sG + i * 1024), 16, 0, 2);
+      } else {
       // 16 bytes per lane: the first half of a lane group's lanes fetches one row of the strip, the second half
       // the next one (64 lanes per row: a wavefront covers two rows of one group; 32: two rows of two groups)
       const int wl = tid & 63;
@@ -182,6 +198,7 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
 #pragma unroll
         for (int k = 0; k < T / 2; ++k)
           __builtin_amdgcn_global_load_lds((global_ptr_t)(c2src + (uint32_t)(2 * k) * c2s), (lds_ptr_t)(sC2 + k * 1024), 16, 0, 2);
+      }
       }
     } else {
 #pragma unroll
@@ -203,19 +220,15 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
       ra[i] = fill_words<Tin, VEC>(true);
       rb[i] = fill_words<Tin, VEC>(false);
       rx[i] = fill_words<Tin, VEC>(false);
-      if (!CLDS) {
-        rc[i] = fill_words<Tin, VEC>(false);
-        rg[i] = fill_words<Tout, VEC>(false);
-      }
+      if (CREG) rc[i] = fill_words<Tin, VEC>(false);
+      if (!CLDS) rg[i] = fill_words<Tout, VEC>(false);
     }
 #pragma unroll
     for (int i = 0; i < T; ++i) {
       if (dok && t0 + i < g.L) {
         ra[i] = load_stream<Tin, VEC>(ab, ao + i * as);
-        if (!CLDS) {
-          rc[i] = load_stream<Tin, VEC>(cb, co + i * cs);
-          rg[i] = load_stream<Tout, VEC>(gb, go + i * gs);
-        }
+        if (CREG) rc[i] = load_stream<Tin, VEC>(cb, co + i * cs);
+        if (!CLDS) rg[i] = load_stream<Tout, VEC>(gb, go + i * gs);
         rb[i] = load_stream<Tin, VEC>(bb, bo + i * bs);
         rx[i] = load_stream<Tin, VEC>(xb, xo + i * xs);
       }
@@ -228,11 +241,11 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
         Words<Tin, VEC> cw = fill_words<Tin, VEC>(false);
         Words<Tout, VEC> gw = fill_words<Tout, VEC>(false);
         if (dok && t0 + i < g.L) {
-          cw = load_stream<Tin, VEC>(cb, co + i * cs);
+          if (!CREG) cw = load_stream<Tin, VEC>(cb, co + i * cs);
           gw = load_stream<Tout, VEC>(gb, go + i * gs);
         }
-        *reinterpret_cast<Words<Tin, VEC>*>(sC + lds_row(i) + lds_lane) = cw;
-        *reinterpret_cast<Words<Tout, VEC>*>(sG + lds_row(i) + lds_lane) = gw;
+        if (!CREG) *reinterpret_cast<Words<Tin, VEC>*>(sC + lds_row(i) + lds_lane) = cw;
+        *reinterpret_cast<Words<Tout, VEC>*>(g_slot(i)) = gw;
         if constexpr (GATED) {
           Words<Tin, VEC> cw2 = fill_words<Tin, VEC>(false);
           if (dok && t0 + i < g.L) cw2 = load_stream<Tin, VEC>(c2b, c2o + i * c2s);
@@ -334,13 +347,10 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   for (int i = T - 1; i >= 0; --i) {
     Words<Tin, VEC> cw;
     Words<Tout, VEC> gw;
-    if (CLDS) {
-      cw = *reinterpret_cast<const Words<Tin, VEC>*>(sC + lds_row(i) + lds_lane);
-      gw = *reinterpret_cast<const Words<Tout, VEC>*>(sG + lds_row(i) + lds_lane);
-    } else {
-      cw = rc[i];
-      gw = rg[i];
-    }
+    if (CREG) cw = rc[i];
+    else cw = *reinterpret_cast<const Words<Tin, VEC>*>(sC + lds_row(i) + lds_lane);
+    if (CLDS) gw = *reinterpret_cast<const Words<Tout, VEC>*>(g_slot(i));
+    else gw = rg[i];
     if constexpr (GATED) {
       const Words<Tin, VEC> cw2 = *reinterpret_cast<const Words<Tin, VEC>*>(sC2 + lds_row(i) + lds_lane);
       float gc[VEC];
@@ -445,7 +455,8 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
 #pragma unroll
     for (int i = 0; i < T; ++i) {
       forget(ra[i]); forget(rb[i]); forget(rx[i]);
-      if (!CLDS) { forget(rc[i]); forget(rg[i]); }
+      if (CREG) forget(rc[i]);
+      if (!CLDS) forget(rg[i]);
     }
     lds_barrier();
 #pragma unroll
@@ -580,13 +591,10 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
     float vdx[VEC], vda[VEC], vdb[VEC], vdc[VEC], vdc2[VEC];
     Words<Tin, VEC> cw;
     Words<Tout, VEC> gw;
-    if (CLDS) {
-      cw = *reinterpret_cast<const Words<Tin, VEC>*>(sC + lds_row(i) + lds_lane);
-      gw = *reinterpret_cast<const Words<Tout, VEC>*>(sG + lds_row(i) + lds_lane);
-    } else {
-      cw = rc[i];
-      gw = rg[i];
-    }
+    if (CREG) cw = rc[i];
+    else cw = *reinterpret_cast<const Words<Tin, VEC>*>(sC + lds_row(i) + lds_lane);
+    if (CLDS) gw = *reinterpret_cast<const Words<Tout, VEC>*>(g_slot(i));
+    else gw = rg[i];
     float zca[VEC], zcb[VEC], sg[VEC];   // GATED: Ca, Cb and sigmoid(Ca) of this step
     if constexpr (GATED) {
       const Words<Tin, VEC> cw2 = *reinterpret_cast<const Words<Tin, VEC>*>(sC2 + lds_row(i) + lds_lane);
@@ -677,7 +685,7 @@ static bool launch_bwd(const BwdArgs& args, int vec, int steps, int threads, boo
     hipLaunchKernelGGL((scan_bwd_kernel<Tin, Tout, V, S, N, C, false, false>), grid, dim3(N), lds, stream, args);    \
     return true;                                                                                                    \
   }
-  if constexpr (sizeof(Tin) == 2 && sizeof(Tout) == 2) {
+  if constexpr (sizeof(Tin) == 2) {
     QSSM_BWD_CASE(4, 8, 256, true)
   }
   QSSM_BWD_CASE(1, 4, 256, false)

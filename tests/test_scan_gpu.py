@@ -176,11 +176,15 @@ def test_lds_resident_operands_and_register_path_agree(gpu, dtype, shape, g_log2
     _check_all(got_reg, ref, TOL[dtype])
 
     x32, a32, b32, c32, dy32 = make_inputs(shape, dtype=dtype, seed=31, out_dtype=torch.float32)
-    got32, _ = run(aligned, out_dtype=torch.float32, gy=dy32)   # forward through LDS, backward (fp32 dy) not
+    # fp32 y and dy: the forward keeps c in LDS, the backward dy alone (16 bytes per lane), c in registers
+    got32, _ = run(aligned, out_dtype=torch.float32, gy=dy32)
     ref32 = oracle_all(x32, a32, b32, c32, dy32)
-    assert_close("y", got32["y"], ref32["y"], 1e-5)
-    for k in ("dx", "da", "db", "dc"):
-        assert_close(k, got32[k], ref32[k], TOL[dtype])
+    got32_reg, _ = run(shifted, out_dtype=torch.float32, gy=dy32)   # and all of it through registers
+    got32_h, _ = run(aligned, out_dtype=torch.float32, gy=dy32, keep_h=True)
+    for got in (got32, got32_reg, got32_h):
+        assert_close("y", got["y"], ref32["y"], 1e-5)
+        for k in ("dx", "da", "db", "dc"):
+            assert_close(k, got[k], ref32[k], TOL[dtype])
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
