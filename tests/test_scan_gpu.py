@@ -1009,3 +1009,31 @@ def test_tiles_that_keep_their_operands_in_the_caches_change_nothing(gpu, hip_li
                                    st(bd), cd.data_ptr(), st(cd), y.data_ptr(), st(y), None, Strides(0, 0),
                                    ck.data_ptr(), ctl.data_ptr(), ctl.numel(), ws.data_ptr(), ws.numel(), 1, stream)
         assert rc == _lib.QSSM_EINVAL
+
+
+def test_seeded_random_shapes_match_the_oracle(gpu):
+    # Shapes, storage types and output types drawn from a fixed seed: whatever geometry the planner picks for them
+    # (strip widths, lanes per row, clusters of 1 to 8, LDS-resident or register operands) must meet the oracle.
+    rng = np.random.default_rng(20240607)
+    pairs = [(torch.float32, torch.float32), (torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16),
+             (torch.float16, torch.float32), (torch.bfloat16, torch.float32)]
+    seen = set()
+    for case in range(36):
+        dtype, out_dtype = pairs[case % len(pairs)]
+        B = int(rng.integers(1, 5))
+        L = int(rng.choice([int(rng.integers(1, 200)), int(rng.integers(200, 3000)), int(rng.integers(3000, 9000))]))
+        D = int(rng.choice([int(rng.integers(1, 40)), 8 * int(rng.integers(1, 80)), 256 * int(rng.integers(1, 4))]))
+        if B * L * D > 6_000_000:
+            L = max(1, 6_000_000 // (B * D))
+        x, a, b, c, dy = make_inputs((B, L, D), dtype=dtype, seed=1000 + case, out_dtype=out_dtype)
+        print(f"case random shape=({B}, {L}, {D}) dtype={dtype} out={out_dtype}", flush=True)
+        got = run_scan_with_grads(scan, x, a, b, c, dy, gpu, out_dtype=out_dtype)
+        assert hip_scan.workspace_status() == 0
+        ref = oracle_all(x, a, b, c, dy)
+        assert_close("y", got["y"], ref["y"], TOL[out_dtype])
+        for k in ("dx", "da", "db", "dc"):
+            assert_close(k, got[k], ref[k], TOL[dtype])
+        align = 8 if D % 8 == 0 else 4 if D % 4 == 0 else 2 if D % 2 == 0 else 1
+        plan = hip_scan.make_plan(B, L, D, dtype, out_dtype, _lib.QSSM_BACKWARD, align, 0)
+        seen.add((plan.vec, plan.g_log2, plan.cluster))
+    assert len({c for _, _, c in seen}) >= 3, seen     # the draw really covers several cluster sizes
