@@ -141,6 +141,45 @@ def _align_elems(tensors: Sequence[Optional[Tensor]], D: int) -> int:
     return 8 if low == 0 or low > 8 else low
 
 
+_ELEM_BYTES = {torch.float32: 4, torch.float16: 2, torch.bfloat16: 2}
+
+
+def _describe(given: Sequence[Optional[Tensor]], fresh: Sequence[Optional[Tensor]], L: int, D: int):
+    """What a launch needs of its tensors, with as few calls into torch as possible (small launches are bound by
+    the host): the caller's tensors made contiguous in their last axis, then strides, base addresses and the
+    alignment in elements (see `_align_elems`) of those and of the freshly allocated, contiguous outputs."""
+    kept, strides, ptrs = [], [], []
+    bits = D
+    for t in given:
+        if t is None:
+            kept.append(None)
+            strides.append(_NO_STRIDE)
+            ptrs.append(None)
+            continue
+        st = t.stride()
+        if st[2] != 1:
+            t = t.contiguous()
+            st = t.stride()
+        ptr = t.data_ptr()
+        es = _ELEM_BYTES[t.dtype]
+        bits |= 1 if ptr % es else (ptr // es) | st[0] | st[1]
+        kept.append(t)
+        strides.append(st)
+        ptrs.append(ptr)
+    out_stride = (L * D, D, 1)
+    for t in fresh:
+        if t is None:
+            strides.append(_NO_STRIDE)
+            ptrs.append(None)
+            continue
+        ptr = t.data_ptr()
+        bits |= (ptr // _ELEM_BYTES[t.dtype]) | out_stride[0]
+        strides.append(out_stride)
+        ptrs.append(ptr)
+    low = bits & -bits
+    return kept, tuple(strides), ptrs, (8 if low == 0 or low > 8 else low)
+
+
 # (device index, stream handle) -> how many `device_counted_launches` contexts are open on it
 _device_counted: Dict[Tuple[int, int], int] = {}
 
@@ -402,12 +441,7 @@ def scan_forward(
             h_final.copy_(h_init) if h_init is not None else h_final.zero_()
         return y, h, (torch.empty((B, 0, D), dtype=torch.float32, device=dev) if want_ckpt else None), 0
 
-    x, a, b = _unit_inner(x), _unit_inner(a), _unit_inner(b)
-    c = _unit_inner(c) if c is not None else None
-    tensors = (x, a, b, c, y, h)
-    strides = tuple(_NO_STRIDE if t is None else t.stride() for t in tensors)
-    ptrs = [0 if t is None else t.data_ptr() for t in tensors]
-    align = _align_elems(tensors, D)
+    (x, a, b, c), strides, ptrs, align = _describe((x, a, b, c), (y, h), L, D)
 
     def make() -> _Launch:
         stride = 0
@@ -483,15 +517,12 @@ def scan_backward(
     if (h is None) == (ckpt is None):
         raise ValueError("pass exactly one of h and ckpt")
 
-    x, a, b, c, dy = (_unit_inner(t) for t in (x, a, b, c, dy))
     if h is not None:
-        h = _unit_inner(h if h.dtype == torch.float32 else h.float())
-    else:
+        if h.dtype != torch.float32:
+            h = h.float()
+    elif not ckpt.is_contiguous():
         ckpt = ckpt.contiguous()
-    tensors = (x, a, b, c, dy, h, *grads)
-    strides = tuple(_NO_STRIDE if t is None else t.stride() for t in tensors)
-    ptrs = [None if t is None else t.data_ptr() for t in tensors]
-    align = _align_elems(tensors, D)
+    (x, a, b, c, dy, h), strides, ptrs, align = _describe((x, a, b, c, dy, h), grads, L, D)
     stride_arg = ckpt_stride if h is None else 0
     out_dtype = dy.dtype
 
