@@ -111,21 +111,6 @@ def kernel_dtypes(in_dtypes: Sequence[torch.dtype], out_dtype: torch.dtype) -> T
     return common, k_out
 
 
-def _unit_inner(t: Tensor) -> Tensor:
-    """A view or copy of `t` whose last axis is contiguous."""
-    return t if t.stride(2) == 1 else t.contiguous()
-
-
-def _strides(t: Optional[Tensor]) -> Strides:
-    if t is None:
-        return Strides(0, 0)
-    return Strides(t.stride(0), t.stride(1))
-
-
-def _ptr(t: Optional[Tensor]) -> Optional[int]:
-    return None if t is None else t.data_ptr()
-
-
 def _align_elems(tensors: Sequence[Optional[Tensor]], D: int) -> int:
     """Largest v in (8, 4, 2, 1) such that D, every stride and every base address (in elements) divide by v."""
     bits = D
