@@ -19,10 +19,11 @@
  *     are passed in elements, so sliced views need no copy.
  *   - Plain pointers and sizes only; every buffer is owned by the caller.  The library never
  *     allocates device memory and never synchronises: kernels are enqueued on `stream`.
+ *     (qssm_scan_forward_static alone works in an array of the library's own; it says so below.)
  *   - Arithmetic is fp32 whatever the storage type; y and the gradients are rounded once.
  *   - Return value: 0 on success, a QSSM_E* code or a hipError_t (> 0) otherwise;
  *     qssm_error_string() describes the last failure on the calling thread.
- *   - Entry points are re-entrant (no global state).
+ *   - Entry points are re-entrant (no global state), with the same one exception.
  */
 #ifndef QUICK_SSM_HIP_H
 #define QUICK_SSM_HIP_H
@@ -70,7 +71,7 @@ typedef struct qssm_plan {
   int32_t in_dtype;       /* x, a, b, c and dx, da, db, dc */
   int32_t out_dtype;      /* y and dy */
   int32_t direction;      /* QSSM_FORWARD / QSSM_BACKWARD */
-  int32_t vec;            /* adjacent columns per lane: 1, 2 or 4 */
+  int32_t vec;            /* adjacent columns per lane: 1, 2 or 4; 8 for a forward over 16-bit storage */
   int32_t steps;          /* consecutive time steps per lane: 4 or 8 */
   int32_t threads;        /* lanes per workgroup: 256, 512 or 1024 */
   int32_t g_log2;         /* log2(lanes per row of a strip) */
