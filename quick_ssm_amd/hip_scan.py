@@ -89,6 +89,10 @@ class _Buffers:
         self.where = where
 
 
+# One entry per (device, raw stream handle, device-counted) ever launched on.  Entries stay until reset_workspaces():
+# a stream handle says nothing about whether its stream still exists, and an entry costs its control block and
+# workspace (tens of MiB for large shapes), so a program that keeps making streams should call reset_workspaces()
+# now and then.
 _buffers: Dict[Tuple[int, int, bool], _Buffers] = {}
 # Buffers a recorded graph still points to, after they have been replaced by larger ones or dropped by
 # reset_workspaces(): kept alive until the process ends, because replaying that graph writes to them.
