@@ -234,22 +234,33 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
       }
     }
     if (CLDS) {
-      // Ragged tile: c and dy go through a register one step at a time (rare, and kept rolled up so
-      // that it does not bring the registers back).
+      // Ragged tile (a partial last strip, or the end of the sequence): c and dy go through registers, half the
+      // tile's steps at a time: rolled up so that it does not bring the registers back, but with the loads of a
+      // half in flight together (one step at a time, a strip of D = 2000 behind seven whole ones cost the backward
+      // 285 us against 219 us for D = 2048).
+      constexpr int HB = T / 2;
 #pragma unroll 1
-      for (int i = 0; i < T; ++i) {
-        Words<Tin, VEC> cw = fill_words<Tin, VEC>(false);
-        Words<Tout, VEC> gw = fill_words<Tout, VEC>(false);
-        if (dok && t0 + i < g.L) {
-          if (!CREG) cw = load_stream<Tin, VEC>(cb, co + i * cs);
-          gw = load_stream<Tout, VEC>(gb, go + i * gs);
+      for (int i0 = 0; i0 < T; i0 += HB) {
+        Words<Tin, VEC> cw[HB], cw2[GATED ? HB : 1];
+        Words<Tout, VEC> gw[HB];
+#pragma unroll
+        for (int u = 0; u < HB; ++u) {
+          const int i = i0 + u;
+          cw[u] = fill_words<Tin, VEC>(false);
+          gw[u] = fill_words<Tout, VEC>(false);
+          if constexpr (GATED) cw2[u] = fill_words<Tin, VEC>(false);
+          if (dok && t0 + i < g.L) {
+            if (!CREG) cw[u] = load_stream<Tin, VEC>(cb, co + i * cs);
+            gw[u] = load_stream<Tout, VEC>(gb, go + i * gs);
+            if constexpr (GATED) cw2[u] = load_stream<Tin, VEC>(c2b, c2o + i * c2s);
+          }
         }
-        if (!CREG) *reinterpret_cast<Words<Tin, VEC>*>(sC + lds_row(i) + lds_lane) = cw;
-        *reinterpret_cast<Words<Tout, VEC>*>(g_slot(i)) = gw;
-        if constexpr (GATED) {
-          Words<Tin, VEC> cw2 = fill_words<Tin, VEC>(false);
-          if (dok && t0 + i < g.L) cw2 = load_stream<Tin, VEC>(c2b, c2o + i * c2s);
-          *reinterpret_cast<Words<Tin, VEC>*>(sC2 + lds_row(i) + lds_lane) = cw2;
+#pragma unroll
+        for (int u = 0; u < HB; ++u) {
+          const int i = i0 + u;
+          if (!CREG) *reinterpret_cast<Words<Tin, VEC>*>(sC + lds_row(i) + lds_lane) = cw[u];
+          *reinterpret_cast<Words<Tout, VEC>*>(g_slot(i)) = gw[u];
+          if constexpr (GATED) *reinterpret_cast<Words<Tin, VEC>*>(sC2 + lds_row(i) + lds_lane) = cw2[u];
         }
       }
     }

@@ -206,18 +206,29 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
       }
     }
     if (CLDS) {
-      // Ragged tile: c goes through a register one step at a time (rare, and kept rolled up so that
-      // it does not bring the sixteen registers back).
+      // Ragged tile (a partial last strip, or the end of the sequence): c goes through registers, half the tile's
+      // steps at a time: rolled up so that it does not bring the registers back, but with the loads of a half in
+      // flight together.
       char* dst = sC + (tid >> 6) * (T * CROW) + lds_lane;
+      constexpr int HB = T / 2;
 #pragma unroll 1
-      for (int i = 0; i < T; ++i) {
-        Words<Tin, VEC> cw = fill_words<Tin, VEC>(false);
-        if (dok && t0 + i < g.L) cw = load_stream<Tin, VEC>(cb, co + i * cs);
-        *reinterpret_cast<Words<Tin, VEC>*>(dst + lds_row(i)) = cw;
-        if constexpr (GATED) {
-          Words<Tin, VEC> cw2 = fill_words<Tin, VEC>(false);
-          if (dok && t0 + i < g.L) cw2 = load_stream<Tin, VEC>(c2b, c2o + i * c2s);
-          *reinterpret_cast<Words<Tin, VEC>*>(dst + (sC2 - sC) + lds_row(i)) = cw2;
+      for (int i0 = 0; i0 < T; i0 += HB) {
+        Words<Tin, VEC> cw[HB], cw2[GATED ? HB : 1];
+#pragma unroll
+        for (int u = 0; u < HB; ++u) {
+          const int i = i0 + u;
+          cw[u] = fill_words<Tin, VEC>(false);
+          if constexpr (GATED) cw2[u] = fill_words<Tin, VEC>(false);
+          if (dok && t0 + i < g.L) {
+            cw[u] = load_stream<Tin, VEC>(cb, co + i * cs);
+            if constexpr (GATED) cw2[u] = load_stream<Tin, VEC>(c2b, c2o + i * c2s);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < HB; ++u) {
+          const int i = i0 + u;
+          *reinterpret_cast<Words<Tin, VEC>*>(dst + lds_row(i)) = cw[u];
+          if constexpr (GATED) *reinterpret_cast<Words<Tin, VEC>*>(dst + (sC2 - sC) + lds_row(i)) = cw2[u];
         }
       }
     }
