@@ -68,6 +68,28 @@ class SSM(nn.Module):
         self.out_proj = proj(self.state_size_dim, hidden_size, True)
         self.pre_norm = RMSNorm(hidden_size, eps=eps, dtype=dtype, device=device) if use_norm else nn.Identity()
 
+    # Below this many elements per projection output a layer's step is bound by launches, not by their work.
+    _BATCHED_PROJECTION_LIMIT = 1 << 23
+
+    def _projections(self, u: torch.Tensor):
+        """The five projection outputs (A, B, C_a, C_b, D order) of the normalised input.
+
+        Small layers (the copy task's 12 x hidden 256: about a thousand launches of a few microseconds each per
+        training step) take one batched GEMM over the five stacked weights instead of five GEMMs, and so one
+        batched GEMM each for the weight and the input gradients instead of ten; the parameters stay the five
+        separate `nn.Linear` modules of the reference.  Large layers keep the separate GEMMs: theirs are efficient
+        already, and the batched input gradient would cost a [5, rows, hidden] intermediate."""
+        S, H = self.state_size_dim, self.hidden_size
+        rows = u.numel() // H
+        if not (u.is_cuda and 0 < rows * S <= self._BATCHED_PROJECTION_LIMIT):
+            return (self.A_proj(u), self.B_proj(u), self.C_proj_a(u), self.C_proj_b(u), self.D_proj(u))
+        w = torch.stack((self.A_proj.weight, self.B_proj.weight, self.C_proj_a.weight, self.C_proj_b.weight,
+                         self.D_proj.weight))                                    # [5, S, H]
+        pre = torch.matmul(u.reshape(1, rows, H), w.transpose(1, 2))             # [5, rows, S]
+        lead = u.shape[:-1]
+        a_pre, b_in, ca, cb, d_pre = (t.view(*lead, S) for t in pre.unbind(0))
+        return (a_pre + self.A_proj.bias, b_in, ca, cb, d_pre)
+
     def gates(self, u: torch.Tensor):
         """The scan's four operands (x, a, b, c) from the normalised input, in `compute_dtype`."""
         forget, drive, out_gate, in_gate = gate_prologue(
@@ -99,7 +121,7 @@ class SSM(nn.Module):
         out_dtype = w_dtype if scan_out_dtype is None else scan_out_dtype
         if backend in ("auto", "hip", "triton") and u.is_cuda and not _scan_interface._HONOR_TILES:
             # 16-bit projections stored as the compute dtype: the activations happen inside the scan's launches
-            pre = (self.A_proj(u), self.B_proj(u), self.C_proj_a(u), self.C_proj_b(u), self.D_proj(u))
+            pre = self._projections(u)
             if _gated.supported(pre, self.compute_dtype, out_dtype, checkpoint):
                 y = _gated.gated_scan(*pre, out_dtype=out_dtype)
             else:

@@ -158,3 +158,35 @@ def test_ssm_layer_with_16_bit_parameters_uses_the_gated_scan_and_matches_the_se
     assert_close("layer dx", dx, dx_ref.double().numpy(), tol)
     for n in g_ref:
         assert_close(f"grad {n}", g[n], g_ref[n].double().numpy(), tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_batched_projection_gemm_equals_the_five_separate_ones(gpu, dtype, monkeypatch):
+    # small layers stack the five projection weights into one batched GEMM; same values and gradients as five
+    # nn.Linear calls, to GEMM rounding, and the parameters (and so the state dict) stay the reference's
+    from quick_ssm_amd.layers import SSM
+
+    torch.manual_seed(1)
+    layer = SSM(hidden_size=64, state_size_mult=4.0, compute_dtype=torch.bfloat16, dtype=dtype).to(gpu)
+    assert sorted(n for n, _ in layer.named_parameters()) == sorted(
+        f"{m}.{p}" for m, ps in (("A_proj", ("weight", "bias")), ("B_proj", ("weight",)), ("C_proj_a", ("weight",)),
+                                 ("C_proj_b", ("weight",)), ("D_proj", ("weight",)), ("out_proj", ("weight", "bias")),
+                                 ("pre_norm", ("weight",))) for p in ps)
+    xin = torch.randn(2, 160, 64, device=gpu).to(dtype)
+    gout = torch.randn(2, 160, 64, device=gpu).to(dtype)
+
+    def run():
+        layer.zero_grad(set_to_none=True)
+        inp = xin.clone().requires_grad_(True)
+        out = layer(inp)
+        out.backward(gout)
+        return out.detach().float().cpu(), inp.grad.float().cpu(), {n: p.grad.float().cpu() for n, p in layer.named_parameters()}
+
+    y_b, dx_b, g_b = run()
+    monkeypatch.setattr(SSM, "_BATCHED_PROJECTION_LIMIT", 0)
+    y_s, dx_s, g_s = run()
+    tol = 1e-4 if dtype == torch.float32 else 3e-2
+    assert_close("layer out", y_b, y_s.double().numpy(), tol)
+    assert_close("layer dx", dx_b, dx_s.double().numpy(), tol)
+    for n in g_s:
+        assert_close(f"grad {n}", g_b[n], g_s[n].double().numpy(), tol)
