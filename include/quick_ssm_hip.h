@@ -365,6 +365,16 @@ QSSM_API int qssm_gates_backward(const void* g_a, const void* g_x, const void* g
                         int64_t rows, int32_t S, int32_t in_dtype, int32_t out_dtype, void* stream);
 
 /*
+ * The same with a row stride `ld_grad` (elements, >= S) for the five gradients, so that they can be written as
+ * column slices of one wide [rows, 5 S] tensor: the gradient of a single GEMM that produced all five projections.
+ */
+QSSM_API int qssm_gates_backward_strided(const void* g_a, const void* g_x, const void* g_c, const void* g_b,
+                                const void* A_pre, int64_t ld_a, const void* Ca, int64_t ld_ca,
+                                const void* Cb, int64_t ld_cb, const void* D_pre, int64_t ld_d,
+                                void* dA_pre, void* dB_in, void* dCa, void* dCb, void* dD_pre, int64_t ld_grad,
+                                int64_t rows, int32_t S, int32_t in_dtype, int32_t out_dtype, void* stream);
+
+/*
  * The scan with the layer's gate activations inside it (quick_ssm/layers.py:76-104 as one launch each way): the
  * operands are the five projection outputs, [B, L, S] with batch and time strides in elements (so they may be
  * column slices of one wide GEMM output), stored as f16 or bf16, and

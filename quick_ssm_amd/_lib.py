@@ -40,6 +40,7 @@ EXPORTED_SYMBOLS = (
     "qssm_scan_gated_backward",
     "qssm_gates_forward",
     "qssm_gates_backward",
+    "qssm_gates_backward_strided",
     "qssm_rmsnorm_forward",
     "qssm_rmsnorm_backward",
     "qssm_copy_bytes",
@@ -176,6 +177,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.qssm_gates_forward.argtypes = [vp, i64] * 5 + [vp] * 4 + [i64, i32, i32, i32, vp]
     lib.qssm_gates_backward.restype = ctypes.c_int
     lib.qssm_gates_backward.argtypes = [vp] * 4 + [vp, i64] * 4 + [vp] * 5 + [i64, i32, i32, i32, vp]
+    lib.qssm_gates_backward_strided.restype = ctypes.c_int
+    lib.qssm_gates_backward_strided.argtypes = [vp] * 4 + [vp, i64] * 4 + [vp] * 5 + [i64, i64, i32, i32, i32, vp]
     lib.qssm_rmsnorm_forward.restype = ctypes.c_int
     lib.qssm_rmsnorm_forward.argtypes = [vp, i64, vp, vp, vp, i64, i32, ctypes.c_float, i32, vp]
     lib.qssm_rmsnorm_backward.restype = ctypes.c_int

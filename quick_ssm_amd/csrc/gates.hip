@@ -82,11 +82,12 @@ __global__ void __launch_bounds__(256) gates_bwd_kernel(const GateBwdArgs p) {
       dCa[v] = gc[v] * zcb[v] * s * (1.0f + zca[v] * (1.0f - s));
       dCb[v] = gc[v] * zca[v] * s;
     }
-    store_f32<Tin, V>(p.dA_pre, o, dA);
-    store_f32<Tin, V>(p.dB_in, o, gx);
-    store_f32<Tin, V>(p.dCa, o, dCa);
-    store_f32<Tin, V>(p.dCb, o, dCb);
-    store_f32<Tin, V>(p.dD_pre, o, dD);
+    const int64_t og = row * p.ld_grad + col;
+    store_f32<Tin, V>(p.dA_pre, og, dA);
+    store_f32<Tin, V>(p.dB_in, og, gx);
+    store_f32<Tin, V>(p.dCa, og, dCa);
+    store_f32<Tin, V>(p.dCb, og, dCb);
+    store_f32<Tin, V>(p.dD_pre, og, dD);
   }
 }
 

@@ -729,17 +729,26 @@ int qssm_gates_backward(const void* g_a, const void* g_x, const void* g_c, const
                         int64_t ld_a, const void* Ca, int64_t ld_ca, const void* Cb, int64_t ld_cb, const void* D_pre,
                         int64_t ld_d, void* dA_pre, void* dB_in, void* dCa, void* dCb, void* dD_pre, int64_t rows,
                         int32_t S, int32_t in_dtype, int32_t out_dtype, void* stream) {
+  return qssm_gates_backward_strided(g_a, g_x, g_c, g_b, A_pre, ld_a, Ca, ld_ca, Cb, ld_cb, D_pre, ld_d, dA_pre, dB_in,
+                                     dCa, dCb, dD_pre, S, rows, S, in_dtype, out_dtype, stream);
+}
+
+int qssm_gates_backward_strided(const void* g_a, const void* g_x, const void* g_c, const void* g_b, const void* A_pre,
+                                int64_t ld_a, const void* Ca, int64_t ld_ca, const void* Cb, int64_t ld_cb,
+                                const void* D_pre, int64_t ld_d, void* dA_pre, void* dB_in, void* dCa, void* dCb,
+                                void* dD_pre, int64_t ld_grad, int64_t rows, int32_t S, int32_t in_dtype,
+                                int32_t out_dtype, void* stream) {
   const int es = dtype_size(in_dtype), os = dtype_size(out_dtype);
   if (es == 0 || os == 0) return fail(QSSM_EINVAL, "unknown dtype code");
   if (rows < 0 || S < 0) return fail(QSSM_EINVAL, "negative dimension");
   if (rows == 0 || S == 0) return 0;
   if (!g_a || !g_x || !g_c || !g_b || !A_pre || !Ca || !Cb || !D_pre || !dA_pre || !dB_in || !dCa || !dCb || !dD_pre)
     return fail(QSSM_EINVAL, "NULL tensor");
-  if (ld_a < S || ld_ca < S || ld_cb < S || ld_d < S) return fail(QSSM_EINVAL, "row stride below S");
+  if (ld_a < S || ld_ca < S || ld_cb < S || ld_d < S || ld_grad < S) return fail(QSSM_EINVAL, "row stride below S");
   GateBwdArgs args{g_a, g_x, g_c, g_b, A_pre, Ca, Cb, D_pre, ld_a, ld_ca, ld_cb, ld_d,
-                   dA_pre, dB_in, dCa, dCb, dD_pre, rows, S};
-  int vec = gate_vec(S, {{A_pre, ld_a}, {Ca, ld_ca}, {Cb, ld_cb}, {D_pre, ld_d}, {dA_pre, S}, {dB_in, S}, {dCa, S},
-                         {dCb, S}, {dD_pre, S}}, es, {g_a, g_x, g_c, g_b}, os);
+                   dA_pre, dB_in, dCa, dCb, dD_pre, rows, S, ld_grad};
+  int vec = gate_vec(S, {{A_pre, ld_a}, {Ca, ld_ca}, {Cb, ld_cb}, {D_pre, ld_d}, {dA_pre, ld_grad}, {dB_in, ld_grad},
+                         {dCa, ld_grad}, {dCb, ld_grad}, {dD_pre, ld_grad}}, es, {g_a, g_x, g_c, g_b}, os);
   if (!launch_gates_any(in_dtype, out_dtype, nullptr, &args, vec, (hipStream_t)stream))
     return fail(QSSM_EINVAL, "gate dtype pair (in=%d, out=%d) is not built", in_dtype, out_dtype);
   hipError_t e = hipGetLastError();

@@ -494,9 +494,10 @@ struct GateBwdArgs {
   const void *g_a, *g_x, *g_c, *g_b;            // [rows, S] contiguous, storage of the scan's operands
   const void *A_pre, *Ca, *Cb, *D_pre;          // [rows, S], row strides in elements
   int64_t ld_a, ld_ca, ld_cb, ld_d;
-  void *dA_pre, *dB_in, *dCa, *dCb, *dD_pre;    // [rows, S] contiguous, storage of the projections
+  void *dA_pre, *dB_in, *dCa, *dCb, *dD_pre;    // [rows, S], storage of the projections, one row stride for all five
   int64_t rows;
   int S;
+  int64_t ld_grad;                               // row stride (elements) of the five gradients: S when contiguous
 };
 
 // One entry per (projection storage, operand storage) pair; exactly one of f, b is non-null.

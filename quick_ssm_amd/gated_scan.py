@@ -23,7 +23,7 @@ import torch
 
 from . import _lib, hip_scan
 from ._lib import Plan, Strides
-from .gates import gate_prologue
+from .gates import gate_prologue, gate_prologue_wide
 
 Tensor = torch.Tensor
 
@@ -77,46 +77,102 @@ def _launch(plan: Plan, dev: torch.device, fn, *args) -> None:
         hip_scan._after_launch(buf, stream, capturing)
 
 
+def _forward_launch(pre: Sequence[Tensor], out_dtype: torch.dtype):
+    """y, the saved states and their spacing for the five projection outputs."""
+    A_pre, B_in, Ca, Cb, D_pre = pre
+    B, L, S = A_pre.shape
+    dev, dtype = A_pre.device, A_pre.dtype
+    # the backward's tile length decides how far apart the saved states are; it takes 16-bit dy only
+    stride = _plan(B, L, S, dtype, dtype, _lib.QSSM_BACKWARD, 0).seg_len
+    plan = _plan(B, L, S, dtype, out_dtype, _lib.QSSM_FORWARD, stride)
+    y = torch.empty((B, L, S), dtype=out_dtype, device=dev)
+    ckpt = torch.empty((B, plan.n_ckpt, S), dtype=torch.float32, device=dev)
+    _launch(plan, dev, _lib.load().qssm_scan_gated_forward,
+            A_pre.data_ptr(), _st(A_pre), B_in.data_ptr(), _st(B_in), Ca.data_ptr(), _st(Ca), Cb.data_ptr(), _st(Cb),
+            D_pre.data_ptr(), _st(D_pre), y.data_ptr(), _st(y), ckpt.data_ptr())
+    return y, ckpt, int(plan.ckpt_stride)
+
+
+def _fits_fused_backward(grad_y: Tensor, dtype: torch.dtype) -> bool:
+    return not (grad_y.dtype != dtype or grad_y.stride(2) != 1 or grad_y.data_ptr() % 16 or (grad_y.stride(0) * 2) % 16
+                or (grad_y.stride(1) * 2) % 16)
+
+
+def _backward_launch(pre: Sequence[Tensor], grad_y: Tensor, ckpt: Tensor, stride: int, grads: Sequence[Tensor]) -> None:
+    """The five projection gradients, written into `grads` (any batch and time strides)."""
+    A_pre, B_in, Ca, Cb, D_pre = pre
+    dA, dB, dCa, dCb, dD = grads
+    B, L, S = A_pre.shape
+    dtype = A_pre.dtype
+    plan = _plan(B, L, S, dtype, dtype, _lib.QSSM_BACKWARD, stride)
+    _launch(plan, A_pre.device, _lib.load().qssm_scan_gated_backward,
+            A_pre.data_ptr(), _st(A_pre), B_in.data_ptr(), _st(B_in), Ca.data_ptr(), _st(Ca), Cb.data_ptr(), _st(Cb),
+            D_pre.data_ptr(), _st(D_pre), grad_y.data_ptr(), _st(grad_y), ckpt.data_ptr(),
+            dA.data_ptr(), _st(dA), dB.data_ptr(), _st(dB), dCa.data_ptr(), _st(dCa), dCb.data_ptr(), _st(dCb),
+            dD.data_ptr(), _st(dD))
+
+
 class _GatedScanFunction(torch.autograd.Function):
     """(A_pre, B_in, Ca, Cb, D_pre) -> y, one HIP launch forward, one backward."""
 
     @staticmethod
     def forward(ctx, A_pre: Tensor, B_in: Tensor, Ca: Tensor, Cb: Tensor, D_pre: Tensor, out_dtype: torch.dtype) -> Tensor:
-        B, L, S = A_pre.shape
-        dev, dtype = A_pre.device, A_pre.dtype
-        # the backward's tile length decides how far apart the saved states are; it takes 16-bit dy only
-        bwd_out = dtype
-        stride = _plan(B, L, S, dtype, bwd_out, _lib.QSSM_BACKWARD, 0).seg_len
-        plan = _plan(B, L, S, dtype, out_dtype, _lib.QSSM_FORWARD, stride)
-        y = torch.empty((B, L, S), dtype=out_dtype, device=dev)
-        ckpt = torch.empty((B, plan.n_ckpt, S), dtype=torch.float32, device=dev)
-        _launch(plan, dev, _lib.load().qssm_scan_gated_forward,
-                A_pre.data_ptr(), _st(A_pre), B_in.data_ptr(), _st(B_in), Ca.data_ptr(), _st(Ca), Cb.data_ptr(), _st(Cb),
-                D_pre.data_ptr(), _st(D_pre), y.data_ptr(), _st(y), ckpt.data_ptr())
+        y, ckpt, stride = _forward_launch((A_pre, B_in, Ca, Cb, D_pre), out_dtype)
         ctx.save_for_backward(A_pre, B_in, Ca, Cb, D_pre, ckpt)
-        ctx.stride, ctx.out_dtype = int(plan.ckpt_stride), out_dtype
+        ctx.stride, ctx.out_dtype = stride, out_dtype
         return y
 
     @staticmethod
     def backward(ctx, grad_y: Tensor):
-        A_pre, B_in, Ca, Cb, D_pre, ckpt = ctx.saved_tensors
-        B, L, S = A_pre.shape
-        dev, dtype = A_pre.device, A_pre.dtype
-        if grad_y.dtype != dtype or grad_y.stride(2) != 1 or grad_y.data_ptr() % 16 or (grad_y.stride(0) * 2) % 16 \
-                or (grad_y.stride(1) * 2) % 16:
+        *pre, ckpt = ctx.saved_tensors
+        B, L, S = pre[0].shape
+        dev, dtype = pre[0].device, pre[0].dtype
+        if not _fits_fused_backward(grad_y, dtype):
             if ctx.out_dtype == dtype:
                 grad_y = grad_y.to(dtype).contiguous()
             else:
                 return _two_pass_backward(ctx, grad_y)
-        plan = _plan(B, L, S, dtype, dtype, _lib.QSSM_BACKWARD, ctx.stride)
         grads = [torch.empty((B, L, S), dtype=dtype, device=dev) for _ in range(5)]
-        dA, dB, dCa, dCb, dD = grads
-        _launch(plan, dev, _lib.load().qssm_scan_gated_backward,
-                A_pre.data_ptr(), _st(A_pre), B_in.data_ptr(), _st(B_in), Ca.data_ptr(), _st(Ca), Cb.data_ptr(), _st(Cb),
-                D_pre.data_ptr(), _st(D_pre), grad_y.data_ptr(), _st(grad_y), ckpt.data_ptr(),
-                dA.data_ptr(), _st(dA), dB.data_ptr(), _st(dB), dCa.data_ptr(), _st(dCa), dCb.data_ptr(), _st(dCb),
-                dD.data_ptr(), _st(dD))
-        return dA, dB, dCa, dCb, dD, None
+        _backward_launch(pre, grad_y, ckpt, ctx.stride, grads)
+        return (*grads, None)
+
+
+def _blocks(wide: Tensor) -> Tuple[Tensor, ...]:
+    S = wide.shape[-1] // 5
+    return tuple(wide[..., k * S:(k + 1) * S] for k in range(5))
+
+
+class _GatedScanWide(torch.autograd.Function):
+    """The same on one wide [B, L, 5 S] tensor whose column blocks are the five projection outputs (one GEMM over the
+    stacked weights): the gradients are written into the blocks of one wide gradient."""
+
+    @staticmethod
+    def forward(ctx, wide: Tensor, out_dtype: torch.dtype) -> Tensor:
+        y, ckpt, stride = _forward_launch(_blocks(wide), out_dtype)
+        ctx.save_for_backward(wide, ckpt)
+        ctx.stride, ctx.out_dtype = stride, out_dtype
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_y: Tensor):
+        wide, ckpt = ctx.saved_tensors
+        dtype = wide.dtype
+        if not _fits_fused_backward(grad_y, dtype):
+            if ctx.out_dtype == dtype:
+                grad_y = grad_y.to(dtype).contiguous()
+            else:
+                with torch.enable_grad():
+                    leaf = wide.detach().requires_grad_(True)
+                    a, x, c, b = gate_prologue_wide(leaf, dtype)
+                k_in, k_out = hip_scan.kernel_dtypes([x.dtype], ctx.out_dtype)
+                dy = grad_y if grad_y.dtype == k_out else grad_y.to(k_out)
+                dx, da, db, dc = hip_scan.scan_backward(x.detach(), a.detach(), b.detach(), c.detach(), dy, ckpt=ckpt,
+                                                        ckpt_stride=ctx.stride)
+                (dwide,) = torch.autograd.grad((a, x, c, b), (leaf,), (da, dx, dc, db))
+                return dwide, None
+        dwide = torch.empty_like(wide, memory_format=torch.contiguous_format)
+        _backward_launch(_blocks(wide), grad_y, ckpt, ctx.stride, _blocks(dwide))
+        return dwide, None
 
 
 def _two_pass_backward(ctx, grad_y: Tensor):
@@ -143,4 +199,10 @@ def gated_scan(A_pre: Tensor, B_in: Tensor, Ca: Tensor, Cb: Tensor, D_pre: Tenso
     return _GatedScanFunction.apply(A_pre, B_in, Ca, Cb, D_pre, out_dtype or A_pre.dtype)
 
 
-__all__ = ["gated_scan", "supported"]
+def gated_scan_wide(wide: Tensor, *, out_dtype: Optional[torch.dtype] = None) -> Tensor:
+    """`gated_scan` on one [B, L, 5 S] tensor holding A_pre, B_in, Ca, Cb, D_pre side by side; call `supported()` on
+    its five blocks first."""
+    return _GatedScanWide.apply(wide, out_dtype or wide.dtype)
+
+
+__all__ = ["gated_scan", "gated_scan_wide", "supported"]

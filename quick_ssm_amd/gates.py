@@ -85,6 +85,66 @@ class _GatePrologue(torch.autograd.Function):
         return tuple(o.view(ctx.shape) for o in outs) + (None,)
 
 
+class _GatePrologueWide(torch.autograd.Function):
+    """The prologue on one wide [.., 5 S] tensor whose column blocks are A_pre, B_in, Ca, Cb, D_pre (the output of a
+    single GEMM over the five stacked projection weights): the kernels read the blocks in place and the backward
+    writes the five gradients into the blocks of one wide gradient, which is what that GEMM's backward wants."""
+
+    @staticmethod
+    def forward(ctx, wide: Tensor, compute_dtype: torch.dtype):
+        S = wide.shape[-1] // 5
+        w2 = _rows(wide, 5 * S)
+        rows = w2.shape[0]
+        ld = w2.stride(0) if rows > 1 else 5 * S
+        es = w2.element_size()
+        outs = [torch.empty((rows, S), dtype=compute_dtype, device=wide.device) for _ in range(4)]
+        with _lib.launch_stream(wide.device) as stream:
+            args = []
+            for k in range(5):
+                args += [w2.data_ptr() + k * S * es, ld]
+            _lib.check(_lib.load().qssm_gates_forward(
+                *args, *[o.data_ptr() for o in outs], rows, S, _CODES[wide.dtype], _CODES[compute_dtype], stream))
+        ctx.save_for_backward(w2)
+        ctx.shape, ctx.out_dtype = wide.shape, compute_dtype
+        lead = wide.shape[:-1]
+        return tuple(o.view(*lead, S) for o in outs)
+
+    @staticmethod
+    def backward(ctx, g_a: Optional[Tensor], g_x: Optional[Tensor], g_c: Optional[Tensor], g_b: Optional[Tensor]):
+        (w2,) = ctx.saved_tensors
+        rows, S = w2.shape[0], w2.shape[1] // 5
+        dev, es = w2.device, w2.element_size()
+        ld = w2.stride(0) if rows > 1 else 5 * S
+
+        def dense(g: Optional[Tensor]) -> Tensor:
+            if g is None:
+                return torch.zeros((rows, S), dtype=ctx.out_dtype, device=dev)
+            g = g.reshape(rows, S)
+            return g if g.is_contiguous() and g.dtype == ctx.out_dtype else g.to(ctx.out_dtype).contiguous()
+
+        gs = [dense(g) for g in (g_a, g_x, g_c, g_b)]
+        dwide = torch.empty((rows, 5 * S), dtype=w2.dtype, device=dev)
+        with _lib.launch_stream(dev) as stream:
+            args = [g.data_ptr() for g in gs]
+            for k in (0, 2, 3, 4):                     # A_pre, Ca, Cb, D_pre
+                args += [w2.data_ptr() + k * S * es, ld]
+            _lib.check(_lib.load().qssm_gates_backward_strided(
+                *args, *[dwide.data_ptr() + k * S * es for k in range(5)], 5 * S, rows, S, _CODES[w2.dtype],
+                _CODES[ctx.out_dtype], stream))
+        return dwide.view(ctx.shape), None
+
+
+def gate_prologue_wide(wide: Tensor, compute_dtype: torch.dtype) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+    """(a, x, c, b) from one [.., 5 S] tensor holding A_pre, B_in, Ca, Cb, D_pre side by side."""
+    if wide.shape[-1] % 5 != 0:
+        raise ValueError("the last axis must hold five blocks of equal width")
+    S = wide.shape[-1] // 5
+    fused = wide.device.type == "cuda" and (wide.dtype, compute_dtype) in _BUILT and wide.numel() > 0
+    if fused:
+        return _GatePrologueWide.apply(wide, compute_dtype)
+    return gates_reference(*(wide[..., k * S:(k + 1) * S] for k in range(5)), compute_dtype)
+
+
 def gate_prologue(A_pre: Tensor, B_in: Tensor, Ca: Tensor, Cb: Tensor, D_pre: Tensor, compute_dtype: torch.dtype
                   ) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
     """(a, x, c, b) in `compute_dtype` from the five projection outputs (all of one shape and dtype).
@@ -103,4 +163,4 @@ def gate_prologue(A_pre: Tensor, B_in: Tensor, Ca: Tensor, Cb: Tensor, D_pre: Te
     return gates_reference(A_pre, B_in, Ca, Cb, D_pre, compute_dtype)
 
 
-__all__ = ["gate_prologue", "gates_reference"]
+__all__ = ["gate_prologue", "gate_prologue_wide", "gates_reference"]

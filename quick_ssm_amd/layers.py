@@ -18,7 +18,7 @@ import torch.nn as nn
 
 from . import gated_scan as _gated
 from . import scan_interface as _scan_interface
-from .gates import gate_prologue
+from .gates import gate_prologue, gate_prologue_wide
 from .norm import rms_norm
 from .scan_interface import scan
 
@@ -71,24 +71,24 @@ class SSM(nn.Module):
     # Below this many elements per projection output a layer's step is bound by launches, not by their work.
     _BATCHED_PROJECTION_LIMIT = 1 << 23
 
-    def _projections(self, u: torch.Tensor):
-        """The five projection outputs (A, B, C_a, C_b, D order) of the normalised input.
+    def _wide_projection(self, u: torch.Tensor) -> Optional[torch.Tensor]:
+        """All five projection outputs as one [.., 5 S] tensor (blocks in A, B, C_a, C_b, D order) from a single GEMM
+        over the concatenated weights, for small layers; None for the others.
 
-        Small layers (the copy task's 12 x hidden 256: about a thousand launches of a few microseconds each per
-        training step) take one batched GEMM over the five stacked weights instead of five GEMMs, and so one
-        batched GEMM each for the weight and the input gradients instead of ten; the parameters stay the five
-        separate `nn.Linear` modules of the reference.  Large layers keep the separate GEMMs: theirs are efficient
-        already, and the batched input gradient would cost a [5, rows, hidden] intermediate."""
+        The copy task's 12 x hidden 256 stack spends a training step on about a thousand launches of a few
+        microseconds each, 194 of them GEMMs: one GEMM forward and two backward per layer instead of five and ten
+        cut both the host's and the GPU's time (the wide tensor's blocks are read in place by the gate kernels, and
+        their gradients are written as blocks of one wide gradient).  The parameters stay the five separate
+        `nn.Linear` modules of the reference.  Large layers keep the separate GEMMs: theirs are efficient already,
+        and the bias gradient over the wide tensor would cost more than it saves."""
         S, H = self.state_size_dim, self.hidden_size
         rows = u.numel() // H
         if not (u.is_cuda and 0 < rows * S <= self._BATCHED_PROJECTION_LIMIT):
-            return (self.A_proj(u), self.B_proj(u), self.C_proj_a(u), self.C_proj_b(u), self.D_proj(u))
-        w = torch.stack((self.A_proj.weight, self.B_proj.weight, self.C_proj_a.weight, self.C_proj_b.weight,
-                         self.D_proj.weight))                                    # [5, S, H]
-        pre = torch.matmul(u.reshape(1, rows, H), w.transpose(1, 2))             # [5, rows, S]
-        lead = u.shape[:-1]
-        a_pre, b_in, ca, cb, d_pre = (t.view(*lead, S) for t in pre.unbind(0))
-        return (a_pre + self.A_proj.bias, b_in, ca, cb, d_pre)
+            return None
+        w = torch.cat((self.A_proj.weight, self.B_proj.weight, self.C_proj_a.weight, self.C_proj_b.weight,
+                       self.D_proj.weight))                                      # [5 S, H]
+        bias = torch.cat((self.A_proj.bias, self.A_proj.bias.new_zeros(4 * S)))
+        return torch.nn.functional.linear(u, w, bias)
 
     def gates(self, u: torch.Tensor):
         """The scan's four operands (x, a, b, c) from the normalised input, in `compute_dtype`."""
@@ -121,11 +121,21 @@ class SSM(nn.Module):
         out_dtype = w_dtype if scan_out_dtype is None else scan_out_dtype
         if backend in ("auto", "hip", "triton") and u.is_cuda and not _scan_interface._HONOR_TILES:
             # 16-bit projections stored as the compute dtype: the activations happen inside the scan's launches
-            pre = self._projections(u)
-            if _gated.supported(pre, self.compute_dtype, out_dtype, checkpoint):
+            wide = self._wide_projection(u)
+            if wide is not None:
+                S = self.state_size_dim
+                pre = tuple(wide[..., k * S:(k + 1) * S] for k in range(5))
+            else:
+                pre = (self.A_proj(u), self.B_proj(u), self.C_proj_a(u), self.C_proj_b(u), self.D_proj(u))
+            if wide is not None and wide.dim() == 3 and _gated.supported(pre, self.compute_dtype, out_dtype, checkpoint):
+                y = _gated.gated_scan_wide(wide, out_dtype=out_dtype)
+            elif _gated.supported(pre, self.compute_dtype, out_dtype, checkpoint):
                 y = _gated.gated_scan(*pre, out_dtype=out_dtype)
             else:
-                forget, drive, out_gate, in_gate = gate_prologue(*pre, self.compute_dtype)
+                if wide is not None:
+                    forget, drive, out_gate, in_gate = gate_prologue_wide(wide, self.compute_dtype)
+                else:
+                    forget, drive, out_gate, in_gate = gate_prologue(*pre, self.compute_dtype)
                 y = scan(x=drive, a=forget, b=in_gate, c=out_gate, block_l=block_l, checkpoint=checkpoint,
                          tile_b=tile_b, tile_d=tile_d, out_dtype=out_dtype, backend=backend)
             return self.out_proj(y.to(w_dtype)) + skip

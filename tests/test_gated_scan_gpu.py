@@ -138,8 +138,9 @@ def test_ssm_layer_with_16_bit_parameters_uses_the_gated_scan_and_matches_the_se
     xin = torch.randn(2, 192, 64).to(dtype)
     gout = torch.randn(2, 192, 64).to(dtype)
     calls = []
-    real = gated_scan.gated_scan
+    real, real_wide = gated_scan.gated_scan, gated_scan.gated_scan_wide
     monkeypatch.setattr(gated_scan, "gated_scan", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    monkeypatch.setattr(gated_scan, "gated_scan_wide", lambda *a, **k: (calls.append(1), real_wide(*a, **k))[1])
 
     def run(mod, inp, backend):
         mod.zero_grad(set_to_none=True)
@@ -190,3 +191,22 @@ def test_batched_projection_gemm_equals_the_five_separate_ones(gpu, dtype, monke
     assert_close("layer dx", dx_b, dx_s.double().numpy(), tol)
     for n in g_s:
         assert_close(f"grad {n}", g_b[n], g_s[n].double().numpy(), tol)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["y16", "y32"])
+def test_gated_scan_on_one_wide_tensor_equals_five_tensors(gpu, out_dtype):
+    # the wide entry (one GEMM's [B, L, 5 S] output in, one wide gradient out): same launches on strided views, so
+    # the same bits as the five-tensor entry; with fp32 y the backward takes the two-pass route in both
+    B, L, S, dtype = 2, 500, 256, torch.bfloat16
+    pre = _projections((B, L, S), dtype, seed=17)
+    dy = torch.randn((B, L, S), generator=torch.Generator().manual_seed(3)).to(out_dtype).to(gpu)
+    leaves = [t.to(gpu).requires_grad_(True) for t in pre]
+    y = gated_scan.gated_scan(*leaves, out_dtype=out_dtype)
+    y.backward(dy)
+    wide = torch.cat(pre, dim=-1).to(gpu).requires_grad_(True)
+    y_w = gated_scan.gated_scan_wide(wide, out_dtype=out_dtype)
+    y_w.backward(dy)
+    assert hip_scan.workspace_status() == 0
+    assert torch.equal(y, y_w)
+    for k, leaf in enumerate(leaves):
+        assert torch.equal(wide.grad[..., k * S:(k + 1) * S], leaf.grad), NAMES[k]

@@ -11,7 +11,7 @@ import torch
 
 from helpers import TOL, assert_close
 from oracle import gates_oracle
-from quick_ssm_amd.gates import gate_prologue, gates_reference
+from quick_ssm_amd.gates import gate_prologue, gate_prologue_wide, gates_reference
 
 pytestmark = pytest.mark.gpu
 
@@ -84,3 +84,29 @@ def test_gate_prologue_saturates_and_falls_back_for_unbuilt_pairs(gpu):
         assert torch.equal(g_, w_)
     with pytest.raises(ValueError):
         gate_prologue(z[0], z[1], z[2], z[3], z[4][:, :4], torch.float32)
+
+
+@pytest.mark.parametrize("in_dtype,out_dtype", [(torch.float32, torch.float16), (torch.bfloat16, torch.bfloat16),
+                                                (torch.float32, torch.float32)], ids=lambda d: str(d).replace("torch.", ""))
+@pytest.mark.parametrize("shape", [(2, 33, 64), (3, 5, 7), (4, 128, 256)], ids=lambda s: "x".join(map(str, s)))
+def test_wide_prologue_equals_the_prologue_on_its_blocks(gpu, in_dtype, out_dtype, shape):
+    # one [.., 5 S] tensor (a single GEMM's output): blocks read in place, gradients written as blocks of one wide
+    # gradient (qssm_gates_backward_strided); same kernels, so the same bits as five separate tensors
+    z = _inputs(shape, in_dtype, seed=7 + sum(shape))
+    gen = torch.Generator().manual_seed(5)
+    g = [torch.randn(*shape, generator=gen).to(out_dtype).to(gpu) for _ in range(4)]
+    leaves = [t.to(gpu).requires_grad_(True) for t in z]
+    outs = gate_prologue(*leaves, out_dtype)
+    torch.autograd.backward(outs, g)
+    wide = torch.cat(z, dim=-1).to(gpu).requires_grad_(True)
+    outs_w = gate_prologue_wide(wide, out_dtype)
+    torch.autograd.backward(outs_w, g)
+    S = shape[-1]
+    for a, b in zip(outs, outs_w):
+        assert torch.equal(a, b)
+    assert wide.grad.shape == wide.shape
+    for k, leaf in enumerate(leaves):
+        assert torch.equal(wide.grad[..., k * S:(k + 1) * S], leaf.grad)
+    ref = gates_oracle.gates_forward_f64(*z)
+    for name, got, want in zip("axcb", outs_w, ref):
+        assert_close(name, got.detach().cpu(), want, TOL[out_dtype])
