@@ -375,7 +375,9 @@ int qssm_plan_scan_tuned(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int3
   // (operands at 5.6 TB/s, with that factor) and its chain (clusters x hand-over): the R with the smaller estimate
   // wins, the smaller R on a tie.  Large launches so get R = 1 or 2, long or narrow ones, whose chains would set
   // the pace, up to 8 (bf16 B=2 L=8192 D=512: forward 84.5 -> 36.3 us, backward 75.6 -> 43.1 us; B=2 L=4096
-  // D=2048: 46.9 -> 36.3 and 86.2 -> 68.2 us).  Single tiles per cluster only with a wide margin (chain within
+  // D=2048: 46.9 -> 36.3 and 86.2 -> 68.2 us), and single long sequences of small width 16 or 32, where the maps
+  // cost 15 - 40 % (B=1 L=16384 D=256: 28.7 -> 19.4 and 55.9 -> 31.6 us; B=1 L=65536 D=512: 94 -> 74 and
+  // 213 -> 158 us).  Single tiles per cluster only with a wide margin (chain within
   // 0.6 of the stream time): bf16 B=16 L=4096 D=2048 forward 233 us against 237, but at B=8 its 64 hand-overs in
   // 116 us would set the pace.
   auto lds_for = [&](int r) -> size_t {
@@ -387,14 +389,18 @@ int qssm_plan_scan_tuned(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int3
   if (tune_r >= 1) {
     cluster = 1 << (tune_r - 1);
   } else if (plan->n_seg > 1) {
-    static const double kMapCost[2][4] = {{-0.02, 0.0, 0.02, 0.035}, {-0.02, 0.0, 0.02, 0.10}};
+    static const double kMapCost[2][6] = {{-0.02, 0.0, 0.02, 0.035, 0.15, 0.40}, {-0.02, 0.0, 0.02, 0.10, 0.30, 0.35}};
     const double hop_us = direction == QSSM_FORWARD ? 2.1 : 1.8;
     const double stream_us = (double)B * L * D * (direction == QSSM_FORWARD ? 4 * es + os : 8 * es + os) / 5.6e6;
     double best = 0.0;
     cluster = 0;
-    for (int k = 0; k < 4; ++k) {
+    // what the kernels that load operands straight into LDS need on top (16-bit storage): clusters beyond 8 must
+    // leave that room, or the launch would fall back to the register-only kernels
+    const size_t staging = es != 2 ? 0 : direction == QSSM_FORWARD ? fwd_c_lds_bytes(threads, steps, vec * es)
+                                                                    : bwd_cg_lds_bytes(threads, steps);
+    for (int k = 0; k < 6; ++k) {
       const int r = 1 << k;
-      if (lds_for(r) > (size_t)kMaxLdsBytes) break;
+      if (lds_for(r) + (k > 3 ? staging : 0) > (size_t)kMaxLdsBytes) break;
       const double chain_us = (double)((plan->n_seg + r - 1) / r) * hop_us;
       if (r == 1 && chain_us > 0.6 * stream_us) continue;
       const double a = stream_us * (1.0 + kMapCost[direction == QSSM_FORWARD ? 0 : 1][k]);

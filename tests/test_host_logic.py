@@ -101,6 +101,8 @@ def test_cluster_size_follows_stream_time_against_chain_time(hip_lib):
     assert clusters(2, 8192, 512, bf, bf) == (8, 8)           # little to stream, long chains: fewest hand-overs
     assert clusters(2, 4096, 2048, bf, bf) == (8, 4)          # the backward pays more per neighbour map
     assert clusters(32, 64, 1024, f16, torch.float32) == (1, 1)   # one tile per chain
+    assert clusters(1, 16384, 256, bf, bf) == (32, 16)        # one long, narrow sequence: the chain is all there is
+    assert clusters(1, 32768, 1024, bf, bf) == (8, 8)         # wider: the maps of 16 tiles would cost more than the hops
 
 
 def test_plan_rejects_bad_arguments(hip_lib):
@@ -275,7 +277,7 @@ def test_plan_invariants_over_random_shapes(hip_lib):
             assert 1 <= (1 << p.g_log2) <= p.threads and p.strip_cols == p.vec << p.g_log2, what
             assert p.seg_len == p.steps * (p.threads >> p.g_log2) and p.seg_len % p.ckpt_stride == 0, what
             assert p.n_strips == -(-D // p.strip_cols) and p.n_seg == -(-L // p.seg_len), what
-            assert p.cluster in (1, 2, 4, 8) and p.n_super == -(-p.n_seg // p.cluster), what
+            assert p.cluster in (1, 2, 4, 8, 16, 32) and p.n_super == -(-p.n_seg // p.cluster), what
             assert 0 < p.lds_bytes <= 64 * 1024, what
             chains = B * p.n_strips
             assert p.control_bytes >= 64 + 64 * chains and p.control_bytes % 256 == 0, what

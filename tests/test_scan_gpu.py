@@ -621,10 +621,11 @@ def test_launch_geometry_does_not_change_results_beyond_rounding(gpu):
     # every lanes-per-row / steps-per-lane geometry must agree with the oracle
     x, a, b, c, dy = make_inputs((2, 1100, 72), seed=8)
     ref = oracle_all(x, a, b, c, dy)
-    dev = [t.to(gpu) for t in (x, a, b, c)]  # L=1100: up to 138 tiles per chain, clusters of 1..8
+    dev = [t.to(gpu) for t in (x, a, b, c)]  # L=1100: up to 138 tiles per chain, clusters of 1..32
     for threads_code, g_log2, steps, cluster_code in [
         (1, 0, 8, 1), (1, 2, 4, 2), (1, 4, 8, 3), (1, 5, 4, 4), (1, 6, 8, 1), (1, 8, 4, 2),
         (2, 3, 8, 2), (2, 6, 4, 3), (2, 9, 8, 1), (3, 4, 4, 2), (3, 6, 8, 3), (3, 5, 4, 4), (3, 10, 4, 1),
+        (1, 4, 4, 5), (1, 5, 8, 6), (1, 2, 4, 6), (2, 4, 4, 5),      # clusters of 16 and 32 tiles: more tiles than lane groups
     ]:
         tune = (g_log2 + 1) | (steps << 8) | (threads_code << 24) | (cluster_code << 28)
         y, _, ckpt, stride = hip_scan.scan_forward(*dev, out_dtype=torch.float32, tune=tune, bwd_tune=tune)
