@@ -324,23 +324,31 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
 
   // ---- sweep 1: fold this lane's T steps into the forward and the reverse affine map ----------
   float A[VEC], Xf[VEC], Xe[VEC];
-  Words<Tin, VEC> za[GATED ? T : 1], zd[GATED ? T : 1];   // GATED: A_pre and D_pre as loaded
+  Words<Tin, VEC> za[GATED ? T : 1], zd[GATED ? T : 1];   // GATED: the derivatives of the two sigmoid gates
 #pragma unroll
   for (int v = 0; v < VEC; ++v) { A[v] = 1.0f; Xf[v] = 0.0f; Xe[v] = 0.0f; }
 #pragma unroll
   for (int i = 0; i < T; ++i) {
     if constexpr (GATED) {
-      // The pre-activations stay beside the gates they turn into: the last sweep wants the derivatives
-      // a (1 - a), b (1 - b) of the unrounded gates (1 - a loses most of its digits when a, close to one, is
-      // first rounded to 16 bits).  Steps past L and columns past D hold the identity (a = 1, b = 0) and keep it.
+      // The derivatives a (1 - a), b (1 - b) of the unrounded gates take the pre-activations' registers, rounded to
+      // the storage type on their own (1 - a loses most of its digits when a, close to one, is first rounded to 16
+      // bits): the last sweep multiplies by them instead of evaluating two more sigmoids per element.  Steps past L
+      // and columns past D hold the identity (a = 1, b = 0) and keep it.
       za[i] = ra[i];
       zd[i] = rb[i];
       if (tile_full || (dok && t0 + i < g.L)) {
-        float ga[VEC], gb[VEC];
+        float ga[VEC], gb[VEC], fa[VEC], fb[VEC];
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) { ga[v] = sigmoid_f(elem(ra[i], v)); gb[v] = sigmoid_f(elem(rb[i], v)); }
+        for (int v = 0; v < VEC; ++v) {
+          ga[v] = sigmoid_f(elem(ra[i], v));
+          gb[v] = sigmoid_f(elem(rb[i], v));
+          fa[v] = ga[v] * (1.0f - ga[v]);
+          fb[v] = gb[v] * (1.0f - gb[v]);
+        }
         ElemBits<Tin>::template set<VEC>(ra[i], ga);
         ElemBits<Tin>::template set<VEC>(rb[i], gb);
+        ElemBits<Tin>::template set<VEC>(za[i], fa);
+        ElemBits<Tin>::template set<VEC>(zd[i], fb);
       }
     }
 #pragma unroll
@@ -637,9 +645,8 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
       round_through<Tin, VEC>(vdc);
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
-        const float av = sigmoid_f(elem(za[i], v)), bv = sigmoid_f(elem(zd[i], v));
-        vda[v] = vda[v] * av * (1.0f - av);
-        vdb[v] = vdb[v] * bv * (1.0f - bv);
+        vda[v] = vda[v] * elem(za[i], v);
+        vdb[v] = vdb[v] * elem(zd[i], v);
         vdc2[v] = vdc[v] * zca[v] * sg[v];
         vdc[v] = vdc[v] * zcb[v] * sg[v] * (1.0f + zca[v] * (1.0f - sg[v]));
       }
