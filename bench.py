@@ -152,14 +152,47 @@ def cpu_baseline(torch, workload, shape, dtype, out_dtype, a_lo, a_span):
     return out
 
 
+def record_traffic(fetch_csv: str, write_csv: str, workload: str) -> int:
+    """Turn two rocprofv3 counter runs of this script (`--pmc FETCH_SIZE`, `--pmc WRITE_SIZE`, each with
+    `--kernel-trace --output-format csv`) into profiles/scan_bwd_<workload>_traffic.json: the backward's HBM bytes
+    per launch, each counter scaled by what it reads for the calibration copy of known size in the same run, tagged
+    with the hash of the kernel sources so that a later run only quotes it while they are unchanged."""
+    import csv
+
+    def mean_kib(path: str, counter: str, kernel: str) -> float:
+        vals = [float(r["Counter_Value"]) for r in csv.DictReader(open(path))
+                if kernel in r["Kernel_Name"] and r["Counter_Name"] == counter]
+        if not vals:
+            raise SystemExit(f"{path}: no {counter} rows for {kernel}")
+        return sum(vals) / len(vals)
+
+    B, L, D, dt_name, out_name = WORKLOADS[workload][:5]
+    n = B * L * D
+    es = {"float32": 4, "float16": 2, "bfloat16": 2}
+    copy_kib = (n * (8 * es[dt_name] + es[out_name]) // 2 // 16) * 16 / 1024      # what the calibration copy moves each way
+    fetch = mean_kib(fetch_csv, "FETCH_SIZE", "scan_bwd") * copy_kib / mean_kib(fetch_csv, "FETCH_SIZE", "copy_kernel")
+    write = mean_kib(write_csv, "WRITE_SIZE", "scan_bwd") * copy_kib / mean_kib(write_csv, "WRITE_SIZE", "copy_kernel")
+    rec = {"kernel": "scan_bwd_kernel", "workload": workload, "traffic_bytes_per_launch": int(fetch * 1024) + int(write * 1024),
+           "fetch_bytes": int(fetch * 1024), "write_bytes": int(write * 1024), "kernel_source_hash": kernel_source_hash(),
+           "source": f"profiles/scan_{workload}_bf16_hbm_traffic.md" if workload == "c1" else "rocprofv3 FETCH_SIZE / WRITE_SIZE"}
+    out = ROOT / "profiles" / f"scan_bwd_{workload}_traffic.json"
+    out.write_text(json.dumps(rec, indent=1))
+    print(json.dumps(rec))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
+    ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="no GPU work: write profiles/scan_bwd_<workload>_traffic.json from two counter_collection.csv files")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
+    if args.record_traffic:
+        return record_traffic(args.record_traffic[0], args.record_traffic[1], args.workload)
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: rows (b, d) of the scan are independent, so more GPUs only shard B or D "
