@@ -89,7 +89,7 @@ static bool aligned_to(const void* p, int64_t sb, int64_t sl, int elem_bytes, in
 static const int kMaxThreads = 1024;
 static const int kMaxLdsBytes = 64 * 1024;
 static const int kCUs = 256;
-static const uint64_t kKeepBytes = 192ull << 20;  // operand bytes a forward leaves in the caches for its backward
+static const uint64_t kKeepBytes = 224ull << 20;  // operand bytes a forward leaves in the caches for its backward
 
 static bool threads_ok(int t) { return t == 256 || t == 512 || t == 1024; }
 
@@ -370,8 +370,9 @@ int qssm_plan_scan_tuned(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int3
 
   // Cluster size R.  Each cluster boundary is one serial hand-over (about 2.1 us forward, 1.8 us backward under
   // load on MI355X) that every chain pays in turn; inside a cluster a tile reads the maps of all earlier tiles,
-  // which costs traffic and LDS (measured against R = 2 on bf16 B=8 L=4096 D=2048: +2 % at R = 4, +3.5 % forward
-  // and +10 % backward at R = 8; R = 1 has no maps at all, -2 %).  A launch takes the longer of its stream time
+  // which costs traffic and LDS (measured against R = 2 on bf16 B=8 L=4096 D=2048: forward +2 % at R = 4 and
+  // +3.5 % at R = 8; backward -0.7 % at R = 4, whose fewer hand-overs outweigh the maps, and +14 % at R = 8; R = 1
+  // has no maps at all, -2 %).  A launch takes the longer of its stream time
   // (operands at 5.6 TB/s, with that factor) and its chain (clusters x hand-over): the R with the smaller estimate
   // wins, the smaller R on a tie.  Large launches so get R = 1 or 2, long or narrow ones, whose chains would set
   // the pace, up to 8 (bf16 B=2 L=8192 D=512: forward 84.5 -> 36.3 us, backward 75.6 -> 43.1 us; B=2 L=4096
@@ -389,7 +390,7 @@ int qssm_plan_scan_tuned(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int3
   if (tune_r >= 1) {
     cluster = 1 << (tune_r - 1);
   } else if (plan->n_seg > 1) {
-    static const double kMapCost[2][6] = {{-0.02, 0.0, 0.02, 0.035, 0.15, 0.40}, {-0.02, 0.0, 0.02, 0.10, 0.30, 0.35}};
+    static const double kMapCost[2][6] = {{-0.02, 0.0, 0.02, 0.035, 0.15, 0.40}, {-0.02, 0.0, -0.005, 0.14, 0.30, 0.35}};
     const double hop_us = direction == QSSM_FORWARD ? 2.1 : 1.8;
     const double stream_us = (double)B * L * D * (direction == QSSM_FORWARD ? 4 * es + os : 8 * es + os) / 5.6e6;
     double best = 0.0;
@@ -423,9 +424,10 @@ int qssm_plan_scan_tuned(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int3
                                           : 0;
   plan->ckpt_elems = (uint64_t)B * plan->n_ckpt * D;
   // The backward starts where the forward ends.  The last tiles of every chain therefore load their operands with
-  // ordinary loads, which leave them in the 256 MiB memory-side cache, as far as three quarters of it reach; the
-  // tiles before them stream past the caches (bf16 B=8 L=4096 D=2048: the last 24 of 64 tiles, backward behind
-  // the forward 229.7 -> 221.2 us).  A launch whose operands fit altogether keeps all of them.
+  // ordinary loads, which leave them in the 256 MiB memory-side cache, as far as seven eighths of it reach; the
+  // tiles before them stream past the caches (bf16 B=8 L=4096 D=2048: the last 28 of 64 tiles; with everything at
+  // fixed addresses the step takes 347.0 us with none kept, 339.7 with 8, 338.2 with 24 or 32, 343.2 with 48).
+  // A launch whose operands fit altogether keeps all of them.
   if (direction == QSSM_FORWARD) {
     const uint64_t per_index = n_chains * (uint64_t)plan->strip_cols * plan->seg_len * 4u * (uint64_t)es;
     const uint64_t keep = kKeepBytes / (per_index > 0 ? per_index : 1);

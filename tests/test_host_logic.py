@@ -56,9 +56,9 @@ def test_plans_are_consistent_and_forward_follows_backward(hip_lib, shape, dtype
             assert p.n_ckpt == -(-L // p.ckpt_stride)
         assert fwd.ckpt_stride == bwd.seg_len == bwd.ckpt_stride
         assert fwd.ckpt_stride % fwd.steps == 0
-        # the forward leaves the operands of its last tiles in the caches, as far as 192 MiB reach; the backward none
+        # the forward leaves the operands of its last tiles in the caches, as far as 224 MiB reach; the backward none
         per_index = B * fwd.n_strips * fwd.strip_cols * fwd.seg_len * 4 * fwd_elem_bytes(dtype)
-        assert fwd.keep_tiles == min(fwd.n_seg, (192 << 20) // per_index) and bwd.keep_tiles == 0
+        assert fwd.keep_tiles == min(fwd.n_seg, (224 << 20) // per_index) and bwd.keep_tiles == 0
         # a backward planned later, with worse alignment, still reads the same saved states
         late = hip_scan.make_plan(B, L, D, dtype, dtype, _lib.QSSM_BACKWARD, 1, bwd.seg_len)
         assert late.ckpt_stride == bwd.seg_len and late.seg_len % late.ckpt_stride == 0
@@ -71,7 +71,7 @@ def fwd_elem_bytes(dtype):
 def test_keep_tiles_of_the_headline_shape(hip_lib):
     bf = torch.bfloat16
     fwd = hip_scan.make_plan(8, 4096, 2048, bf, bf, _lib.QSSM_FORWARD, 8, 32)
-    assert (fwd.vec, fwd.n_seg, fwd.keep_tiles) == (8, 64, 24)
+    assert (fwd.vec, fwd.n_seg, fwd.keep_tiles) == (8, 64, 28)
 
 
 def test_sixteen_bytes_per_lane_only_where_it_pays(hip_lib):
@@ -95,7 +95,7 @@ def test_cluster_size_follows_stream_time_against_chain_time(hip_lib):
         fwd = hip_scan.make_plan(B, L, D, dt, odt, _lib.QSSM_FORWARD, 8, bwd.seg_len)
         return fwd.cluster, bwd.cluster
 
-    assert clusters(8, 4096, 2048, bf, bf) == (2, 2)          # chain and stream in balance
+    assert clusters(8, 4096, 2048, bf, bf) == (2, 4)          # chain and stream in balance; the backward's hops cost more than its maps
     assert clusters(16, 4096, 2048, bf, bf) == (1, 1)         # stream time dwarfs the chain: no maps at all
     assert clusters(1, 65536, 4096, f16, f16) == (4, 4)       # very long chains
     assert clusters(2, 8192, 512, bf, bf) == (8, 8)           # little to stream, long chains: fewest hand-overs
