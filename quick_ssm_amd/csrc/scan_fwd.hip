@@ -151,12 +151,13 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
     // Loads that differ in nothing but their cache policy look alike to the optimizer, which would hoist one
     // (ordinary) copy in front of the branch; a fence at the head of one flavour keeps them apart.
     if constexpr (KEEP) asm volatile("" ::: "memory");
+    // one tensor after the other rather than step by step: a hair faster (0.4 us of 125 on the headline shape)
 #pragma unroll
-    for (int i = 0; i < T; ++i) {
-      ra[i] = load_stream<Tin, VEC, KEEP>(ab, ao + i * as);
-      rb[i] = load_stream<Tin, VEC, KEEP>(bb, bo + i * bs);
-      rx[i] = load_stream<Tin, VEC, KEEP>(xb, xo + i * xs);
-    }
+    for (int i = 0; i < T; ++i) ra[i] = load_stream<Tin, VEC, KEEP>(ab, ao + i * as);
+#pragma unroll
+    for (int i = 0; i < T; ++i) rb[i] = load_stream<Tin, VEC, KEEP>(bb, bo + i * bs);
+#pragma unroll
+    for (int i = 0; i < T; ++i) rx[i] = load_stream<Tin, VEC, KEEP>(xb, xo + i * xs);
     if (CLDS && WIDE) {
       char* dst = sC + (tid >> 6) * (T * CROW);
 #pragma unroll
