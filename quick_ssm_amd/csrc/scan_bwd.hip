@@ -189,11 +189,13 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
       const int half = (wl >> (g.g_log2 - 1)) & 1, piece = wl & ((G >> 1) - 1);
       const char* csrc = cb + (uint32_t)(j * T + half) * cs + (uint32_t)piece * 16u;
       const char* gsrc = gb + (uint32_t)(j * T + half) * gs + (uint32_t)piece * 16u;
+      // one tensor after the other here as well (1.8 us of 211 on the headline shape against c and dy in turn)
 #pragma unroll
-      for (int k = 0; k < T / 2; ++k) {
+      for (int k = 0; k < T / 2; ++k)
         __builtin_amdgcn_global_load_lds((global_ptr_t)(csrc + (uint32_t)(2 * k) * cs), (lds_ptr_t)(sC + k * 1024), 16, 0, 2);
+#pragma unroll
+      for (int k = 0; k < T / 2; ++k)
         __builtin_amdgcn_global_load_lds((global_ptr_t)(gsrc + (uint32_t)(2 * k) * gs), (lds_ptr_t)(sG + k * 1024), 16, 0, 2);
-      }
       if constexpr (GATED) {
         const char* c2src = c2b + (uint32_t)(j * T + half) * c2s + (uint32_t)piece * 16u;
 #pragma unroll
