@@ -5,6 +5,7 @@ storage, the oracle being float64 arithmetic on the same stored inputs.  fp32 ca
 to the reference tests' own allclose(rtol=1e-3, atol=1e-5) against the fp32 sequential recurrence.
 """
 import json
+import os
 from pathlib import Path
 
 import numpy as np
@@ -1015,11 +1016,13 @@ def test_tiles_that_keep_their_operands_in_the_caches_change_nothing(gpu, hip_li
 def test_seeded_random_shapes_match_the_oracle(gpu):
     # Shapes, storage types and output types drawn from a fixed seed: whatever geometry the planner picks for them
     # (strip widths, lanes per row, clusters of 1 to 8, LDS-resident or register operands) must meet the oracle.
+    # QSSM_RANDOM_CASES=n draws n cases instead of 36 (the first 36 stay the same ones).
+    n_cases = int(os.environ.get("QSSM_RANDOM_CASES", "36"))
     rng = np.random.default_rng(20240607)
     pairs = [(torch.float32, torch.float32), (torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16),
              (torch.float16, torch.float32), (torch.bfloat16, torch.float32)]
     seen = set()
-    for case in range(36):
+    for case in range(n_cases):
         dtype, out_dtype = pairs[case % len(pairs)]
         B = int(rng.integers(1, 5))
         L = int(rng.choice([int(rng.integers(1, 200)), int(rng.integers(200, 3000)), int(rng.integers(3000, 9000))]))
