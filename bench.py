@@ -28,6 +28,8 @@ if str(ROOT) not in sys.path:
     sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak, 8 TB/s
+SETTLE_MS = 30.0        # untimed load in front of the first measurement (see main)
+IDLE_MS = 250.0         # idle spell in front of the `after_idle` figure
 
 WORKLOADS = {
     # name: (B, L, D, operand dtype, y/dy dtype, a_lo, a_span, block_l, description)
@@ -247,10 +249,19 @@ def main() -> int:
         with torch.autograd.set_multithreading_enabled(False):
             y.backward(gy)
 
-    # ---- the two kernels on their own, through the C ABI -------------------------------------------
-    # Measured first: the device's power management takes some 10 ms of load to settle (launches right after an
-    # idle spell run 3-5 % slow), and the whole-step figure below should be the settled one a training job sees.
+    # ---- everything the run needs exists before the first measured launch ------------------------
+    # An allocation of this size is milliseconds of idle GPU, and an idle spell of 10 ms or more is followed by
+    # about 10 ms in which the device runs the same launches up to 8 % slower (it starts fast, sags after 1-2 ms
+    # and recovers; profiles/device_settle_timeline.md): every leg below therefore follows the one before without
+    # a pause, behind a run of untimed launches that outlasts that spell, and what is reported is the settled
+    # rate a job that keeps the device busy sees.  `after_idle` at the end reports the other case.
     xd, ad, bd, cd = (t.detach() for t in leaves)
+    nb = (bwd_bytes // 2 // 16) * 16
+    src = torch.empty(nb, dtype=torch.uint8, device=dev)
+    dst = torch.empty(nb, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    lib = _lib.load()
+    step()          # plans, argument blocks, control block, workspace and the allocator's blocks for y and the gradients
     with torch.no_grad():
         _, _, ckpt, stride = hip_scan.scan_forward(xd, ad, bd, cd, out_dtype=out_dtype)
         detached = [tuple(t.detach() for t in ops) + (gy,) for ops, gy in sets]
@@ -265,25 +276,35 @@ def main() -> int:
             turn[0] += 1
             hip_scan.scan_backward(xs, as_, bs, cs, gy, ckpt=ckpt, ckpt_stride=stride)
 
-        # each launch repeated on its own (a forward then finds the operands its predecessor kept in the caches for
-        # a backward that never came, so this figure flatters it), and the two in turn as a step runs them
-        fwd_alone_ms = event_time_ms(torch, fwd_once, args.steps, args.warmup)
-        bwd_alone_ms = event_time_ms(torch, bwd_once, args.steps, args.warmup)
-
         def fwd_same_set():
             xs, as_, bs, cs, _ = detached[turn[0] % n_sets]
             hip_scan.scan_forward(xs, as_, bs, cs, out_dtype=out_dtype)
 
-        fwd_ms, bwd_ms = alternating_times_ms(torch, fwd_same_set, bwd_once, args.steps, args.warmup)
+        # untimed: the two launches in turn until the device has been busy for SETTLE_MS without a pause
+        torch.cuda.synchronize()
+        t_settle = time.perf_counter()
+        settle_pairs = 0
+        while (time.perf_counter() - t_settle) * 1e3 < SETTLE_MS:
+            for _ in range(8):
+                fwd_same_set()
+                bwd_once()
+            settle_pairs += 8
+            torch.cuda.synchronize()
+
+        # ---- the two kernels on their own, through the C ABI ---------------------------------------
+        # each launch repeated on its own (a forward then finds the operands its predecessor kept in the caches for
+        # a backward that never came, so this figure flatters it), and the two in turn as a step runs them
+        fwd_alone_ms = event_time_ms(torch, fwd_once, args.steps, args.warmup)
+        bwd_alone_ms = event_time_ms(torch, bwd_once, args.steps, args.warmup)
         # achievable ceiling on this box: a plain copy of the same number of bytes as the backward moves
-        nb = (bwd_bytes // 2 // 16) * 16
-        src = torch.empty(nb, dtype=torch.uint8, device=dev)
-        dst = torch.empty(nb, dtype=torch.uint8, device=dev)
-        stream = torch.cuda.current_stream().cuda_stream
-        lib = _lib.load()
         copy_ms = event_time_ms(torch, lambda: lib.qssm_copy_bytes(dst.data_ptr(), src.data_ptr(), nb, stream),
                                 args.steps, args.warmup)
-        del src, dst
+        # the forward without its cache policy (every operand streamed past the caches) and the backward behind it:
+        # what the pair costs when other work runs between a layer's forward and its backward
+        hip_scan.set_forward_keep(False)
+        fwd_nokeep_ms, bwd_nokeep_ms = alternating_times_ms(torch, fwd_same_set, bwd_once, args.steps, args.warmup)
+        hip_scan.set_forward_keep(True)
+        fwd_ms, bwd_ms = alternating_times_ms(torch, fwd_same_set, bwd_once, args.steps, args.warmup)
     # ---- whole step through the public API: W warm-ups, then exactly K timed steps ---------------
     for _ in range(args.warmup):
         step()
@@ -298,6 +319,15 @@ def main() -> int:
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     gpu_ms = ev0.elapsed_time(ev1) / args.steps
     ms_per_step = wall_ms
+
+    # the same K steps right after an idle spell, no warm-up: what a job that leaves the device idle between steps sees
+    time.sleep(IDLE_MS * 1e-3)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    after_idle_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    del src, dst
 
     status = hip_scan.workspace_status()
     align = hip_scan._align_elems([xd, ad, bd, cd, dy], D)   # what the timed launches were planned with
@@ -365,6 +395,15 @@ def main() -> int:
         },
         "workspace_status": status,
         "rotated_operand_sets": n_sets,
+        # untimed fwd+bwd pairs in front of every measurement (the device settles for about 10 ms after an idle spell)
+        "settle": {"ms": SETTLE_MS, "pairs": settle_pairs},
+        # the same K steps begun right after an idle spell, no warm-up
+        "after_idle": {"idle_ms": IDLE_MS, "steps": args.steps, "ms_per_step": after_idle_ms,
+                       "pct_of_hbm_peak": 100.0 * step_bytes / (after_idle_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
+        # the two launches in turn with every operand of the forward streamed past the caches (plan.keep_tiles = 0):
+        # the pair's cost when other work runs between a forward and its backward
+        "without_cache_policy": {"fwd_ms": fwd_nokeep_ms, "bwd_ms": bwd_nokeep_ms,
+                                 "pct_of_hbm_peak": 100.0 * step_bytes / ((fwd_nokeep_ms + bwd_nokeep_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, args.workload, shape, dtype, out_dtype, a_lo, a_span)

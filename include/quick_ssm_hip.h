@@ -41,7 +41,7 @@ extern "C" {
 #define QSSM_API
 #endif
 
-#define QSSM_VERSION 100 /* major*10000 + minor*100 + patch */
+#define QSSM_VERSION 200 /* major*10000 + minor*100 + patch; 0.2.0: qssm_plan_scan without `tune`, qssm_plan.keep_tiles */
 
 /* storage types */
 #define QSSM_F32 0
@@ -456,6 +456,17 @@ QSSM_API int qssm_rmsnorm_backward(const void* dy, int64_t ld_dy, const void* x,
  * counters and the achievable-bandwidth ceiling are calibrated by the benchmark.
  */
 QSSM_API int qssm_copy_bytes(void* dst, const void* src, uint64_t bytes, void* stream);
+
+/*
+ * Host-side mirror of the launch counter that launches with epoch argument 0 keep in their control
+ * block (no GPU work): for a counter reading `count` before a launch, `*flag` is the flag value the
+ * launch tags its words with, `*next` the reading afterwards, and `*wipes` whether the launch's
+ * prologue clears the whole scratch array first (only qssm_scan_forward_static, `static_scratch`
+ * nonzero, ever does).  No counterpart in the reference; it lets a caller, or a test, follow the
+ * numbering across its wrap without driving a GPU through 2^32 launches.
+ */
+QSSM_API int qssm_launch_count_step(uint32_t count, int32_t static_scratch, uint32_t* flag, uint32_t* next,
+                                    int32_t* wipes);
 
 #ifdef __cplusplus
 }

@@ -14,6 +14,8 @@ from typing import Optional
 LIB_NAME = "libquick_ssm_hip.so"
 LIB_PATH = Path(__file__).resolve().parent / LIB_NAME
 
+# The QSSM_VERSION of include/quick_ssm_hip.h this binding was written against (same minor version = same ABI).
+QSSM_VERSION = 200
 QSSM_F32, QSSM_F16, QSSM_BF16 = 0, 1, 2
 QSSM_FORWARD, QSSM_BACKWARD = 0, 1
 QSSM_RMSNORM_MIN_PARTIAL_ROWS = 8
@@ -44,6 +46,7 @@ EXPORTED_SYMBOLS = (
     "qssm_rmsnorm_forward",
     "qssm_rmsnorm_backward",
     "qssm_copy_bytes",
+    "qssm_launch_count_step",
 )
 
 
@@ -185,6 +188,9 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.qssm_rmsnorm_backward.argtypes = [vp, i64, vp, i64, vp, vp, vp, vp, vp, i32, i64, i32, ctypes.c_float, i32, vp]
     lib.qssm_copy_bytes.restype = ctypes.c_int
     lib.qssm_copy_bytes.argtypes = [vp, vp, u64, vp]
+    lib.qssm_launch_count_step.restype = ctypes.c_int
+    lib.qssm_launch_count_step.argtypes = [ctypes.c_uint32, i32, ctypes.POINTER(ctypes.c_uint32),
+                                           ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(i32)]
 
 
 def is_built() -> bool:
@@ -204,6 +210,12 @@ def load() -> ctypes.CDLL:
                     "Run `python -m quick_ssm_amd.build` (needs hipcc). There is no other device path."
                 )
             lib = ctypes.CDLL(os.fspath(LIB_PATH))
+            lib.qssm_version.restype = ctypes.c_int
+            built = int(lib.qssm_version())
+            if built // 100 != QSSM_VERSION // 100:
+                raise RuntimeError(
+                    f"{LIB_PATH} was built from version {built} of the C ABI, this package binds version "
+                    f"{QSSM_VERSION}: the argument lists differ. Rebuild with `python -m quick_ssm_amd.build`.")
             _declare(lib)
             _lib = lib
     return _lib

@@ -144,8 +144,7 @@ static bool tile_span_ok(const qssm_plan* pl, const void* p, int64_t sb, int64_t
 // the library's own scratch array wraps earlier, after its workspace has been wiped).
 static const unsigned kCountWrapAt = 0xfffffffeu;
 __global__ void count_launch_kernel(unsigned* count, unsigned reset_at) {
-  const unsigned cur = *count;
-  *count = cur >= reset_at ? 0u : cur + 1u;
+  *count = launch_count_next(*count, reset_at);
 }
 
 static void fill_geometry(Geometry* g, const qssm_plan* pl, void* control, void* workspace, uint32_t epoch) {
@@ -825,8 +824,9 @@ static std::mutex g_scratch_mutex;
 // an old launch can ever carry the flag value of a new one.  Every workgroup reads the count before anyone
 // rewrites the word beside it with the same value.
 __global__ void __launch_bounds__(256) scratch_prologue_kernel(uint4* scratch, uint64_t control16, uint64_t total16) {
+  static_assert(kLaunchCountOffset == 4, "the count is the second word of the control block's first 16 bytes");
   const unsigned count = reinterpret_cast<const unsigned*>(scratch)[kLaunchCountOffset / 4];
-  const uint64_t n16 = count >= kScratchWipeAt ? total16 : control16;
+  const uint64_t n16 = scratch_wipe_due(count, kScratchWipeAt) ? total16 : control16;
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride)
     scratch[i] = i == 0 ? make_uint4(0u, count, 0u, 0u) : make_uint4(0u, 0u, 0u, 0u);
@@ -877,6 +877,15 @@ extern "C" int qssm_scan_forward_static(const qssm_plan* plan, const void* x, qs
 }
 
 extern "C" {
+
+int qssm_launch_count_step(uint32_t count, int32_t static_scratch, uint32_t* flag, uint32_t* next, int32_t* wipes) {
+  if (flag == nullptr || next == nullptr || wipes == nullptr) return fail(QSSM_EINVAL, "NULL argument");
+  const unsigned reset_at = static_scratch ? kScratchWipeAt : kCountWrapAt;
+  *flag = count + 1u;
+  *next = launch_count_next(count, reset_at);
+  *wipes = static_scratch && scratch_wipe_due(count, kScratchWipeAt) ? 1 : 0;
+  return 0;
+}
 
 int qssm_copy_bytes(void* dst, const void* src, uint64_t bytes, void* stream) {
   if (bytes == 0) return 0;

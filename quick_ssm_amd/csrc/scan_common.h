@@ -399,9 +399,20 @@ __device__ __forceinline__ unsigned claim_ticket(unsigned* tickets, int chain, i
   return tk;
 }
 
+// Status codes are bits (1: a tile gave up waiting, 2: the control block was dirty on entry) and accumulate.
 __device__ __forceinline__ void raise_status(int* status, int code) {
-  __hip_atomic_store(status, code, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_fetch_or(status, code, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+
+// The launch count kept in the control block (device-counted epochs).  A launch uses flag value count + 1; the
+// counting kernel behind it stores launch_count_next(count, reset_at).  The count never takes the value whose
+// successor is zero: from `reset_at` on it starts again at zero, and a caller that lets it do so must have
+// cleared every word of the old numbering first (scratch_wipe_due: the library's own scratch array does that in
+// the prologue of the launch that finds the count at or beyond its wipe mark).
+__host__ __device__ inline unsigned launch_count_next(unsigned count, unsigned reset_at) {
+  return count >= reset_at ? 0u : count + 1u;
+}
+__host__ __device__ inline bool scratch_wipe_due(unsigned count, unsigned wipe_at) { return count >= wipe_at; }
 
 // ---- kernel arguments -----------------------------------------------------------------------
 

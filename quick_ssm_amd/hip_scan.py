@@ -82,7 +82,11 @@ class _Buffers:
         self.epoch = 0
         self.ctl_ptr = self.ctl_size = self.ws_ptr = self.ws_size = 0
         self.captured = False          # a graph holds these addresses: never free or move them
+        # The status word is copied here by a raw asynchronous copy that torch's pinned-memory allocator knows
+        # nothing about: the block must never go back to it, or a copy still queued when the entry is dropped
+        # would land in somebody else's tensor.  Four bytes per (device, stream) ever used.
         self.pinned = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+        _pinned_words.append(self.pinned)
         self.seen = ctypes.c_int32.from_address(self.pinned.data_ptr())
         self.since_check = 0
         self.device = device
@@ -94,6 +98,7 @@ class _Buffers:
 # workspace (tens of MiB for large shapes), so a program that keeps making streams should call reset_workspaces()
 # now and then.
 _buffers: Dict[Tuple[int, int, bool], _Buffers] = {}
+_pinned_words: List[Tensor] = []
 # Buffers a recorded graph still points to, after they have been replaced by larger ones or dropped by
 # reset_workspaces(): kept alive until the process ends, because replaying that graph writes to them.
 _retired: List[Tensor] = []
@@ -210,30 +215,35 @@ class device_counted_launches:
 def _grow_buffers(key: Tuple[int, int, bool], device: torch.device, need_c: int, need_w: int, capturing: bool) -> _Buffers:
     """Slow path of `_launch_buffers`: first use of a (device, stream), a larger shape, or a used-up numbering."""
     with _ws_lock:
-        buf = _buffers.get(key)
-        grow_c = buf is None or buf.control is None or buf.ctl_size < need_c
-        grow_w = grow_c or buf.workspace is None or buf.ws_size < need_w or buf.epoch >= _EPOCH_MAX
-        if capturing and grow_w:   # before anything is allocated: an allocation would spoil the recording
-            raise RuntimeError(
-                "quick_ssm_amd: a scan launch being recorded into a graph cannot allocate its control block and "
-                "workspace; run the same work once inside `hip_scan.device_counted_launches()` on this stream first")
-        if buf is None:
-            buf = _Buffers(device, f"device {key[0]}, stream {key[1]:#x}")
-        if buf.captured and grow_w:
-            # a recorded graph points at the old pair: keep it alive and untouched, new launches get a new pair
-            _retired.extend(t for t in (buf.control, buf.workspace) if t is not None)
-            buf.captured = False
-            grow_c = True
-        if grow_c:
-            # a new control block restarts the device-side count: the workspace must not keep words of the old numbering
-            buf.control = torch.zeros(max(1 << 16, 1 << (need_c - 1).bit_length()), dtype=torch.uint8, device=device)
-            buf.ctl_ptr, buf.ctl_size = buf.control.data_ptr(), buf.control.numel()
-        if grow_w:
-            buf.workspace = torch.zeros(max(1 << 20, 1 << (need_w - 1).bit_length()), dtype=torch.uint8, device=device)
-            buf.ws_ptr, buf.ws_size = buf.workspace.data_ptr(), buf.workspace.numel()
-            buf.epoch = 0
-        _buffers[key] = buf
-        return buf
+        return _grow_buffers_locked(key, device, need_c, need_w, capturing)
+
+
+def _grow_buffers_locked(key: Tuple[int, int, bool], device: torch.device, need_c: int, need_w: int, capturing: bool) -> _Buffers:
+    """`_grow_buffers` for a caller that holds `_ws_lock`."""
+    buf = _buffers.get(key)
+    grow_c = buf is None or buf.control is None or buf.ctl_size < need_c
+    grow_w = grow_c or buf.workspace is None or buf.ws_size < need_w or buf.epoch >= _EPOCH_MAX
+    if capturing and grow_w:   # before anything is allocated: an allocation would spoil the recording
+        raise RuntimeError(
+            "quick_ssm_amd: a scan launch being recorded into a graph cannot allocate its control block and "
+            "workspace; run the same work once inside `hip_scan.device_counted_launches()` on this stream first")
+    if buf is None:
+        buf = _Buffers(device, f"device {key[0]}, stream {key[1]:#x}")
+    if buf.captured and grow_w:
+        # a recorded graph points at the old pair: keep it alive and untouched, new launches get a new pair
+        _retired.extend(t for t in (buf.control, buf.workspace) if t is not None)
+        buf.captured = False
+        grow_c = True
+    if grow_c:
+        # a new control block restarts the device-side count: the workspace must not keep words of the old numbering
+        buf.control = torch.zeros(max(1 << 16, 1 << (need_c - 1).bit_length()), dtype=torch.uint8, device=device)
+        buf.ctl_ptr, buf.ctl_size = buf.control.data_ptr(), buf.control.numel()
+    if grow_w:
+        buf.workspace = torch.zeros(max(1 << 20, 1 << (need_w - 1).bit_length()), dtype=torch.uint8, device=device)
+        buf.ws_ptr, buf.ws_size = buf.workspace.data_ptr(), buf.workspace.numel()
+        buf.epoch = 0
+    _buffers[key] = buf
+    return buf
 
 
 def _recover(buf: _Buffers, stream: int) -> int:
@@ -244,10 +254,11 @@ def _recover(buf: _Buffers, stream: int) -> int:
         _lib.check(lib.qssm_zero_fill(buf.ws_ptr, buf.ws_size, stream))
         out = ctypes.c_int32(0)
         _lib.check(lib.qssm_control_status(buf.ctl_ptr, stream, ctypes.byref(out)))   # waits: copies in flight have landed
-    status = int(buf.seen.value)
-    buf.seen.value = 0
-    buf.epoch = 0
-    buf.since_check = 0
+    with _ws_lock:
+        status = int(buf.seen.value)
+        buf.seen.value = 0
+        buf.epoch = 0
+        buf.since_check = 0
     return status
 
 
@@ -267,26 +278,36 @@ def _launch_buffers(device: torch.device, dev_index: int, stream: int, need_c: i
     capturing = torch._C._cuda_isCurrentStreamCapturing()
     on_device = capturing or ((dev_index, stream) in _device_counted)
     key = (dev_index, stream, on_device)
-    buf = _buffers.get(key)
-    if buf is None or buf.ctl_size < need_c or buf.ws_size < need_w or buf.epoch >= _EPOCH_MAX:
-        buf = _grow_buffers(key, device, need_c, max(need_w, 256), capturing)
-    if buf.seen.value != 0 and not capturing:
+    # Looking the buffers up and taking the next number is one step under the lock: the forward of the next step on
+    # the caller's thread and a backward on autograd's thread may launch on one stream at the same time, and two
+    # launches with one number would read each other's words as their own.
+    with _ws_lock:
+        buf = _buffers.get(key)
+        if buf is None or buf.ctl_size < need_c or buf.ws_size < need_w or buf.epoch >= _EPOCH_MAX:
+            buf = _grow_buffers_locked(key, device, need_c, max(need_w, 256), capturing)
+        failed = buf.seen.value != 0 and not capturing
+        epoch = 0
+        if not failed:
+            if capturing:
+                buf.captured = True
+            if not on_device:
+                buf.epoch += 1
+                epoch = buf.epoch
+    if failed:
         raise ScanLaunchError(_recover(buf, stream), buf.where)
-    if capturing:
-        buf.captured = True
-    if on_device:
-        return buf, 0, capturing
-    buf.epoch += 1
-    return buf, buf.epoch, capturing
+    return buf, epoch, capturing
 
 
 def _after_launch(buf: _Buffers, stream: int, capturing: bool) -> None:
     """Every `_check_every`-th launch: ask for the status word, to be looked at before a later launch."""
     if _check_every <= 0 or capturing:
         return
-    buf.since_check += 1
-    if buf.since_check >= _check_every:
-        buf.since_check = 0
+    with _ws_lock:
+        buf.since_check += 1
+        due = buf.since_check >= _check_every
+        if due:
+            buf.since_check = 0
+    if due:
         _lib.check(_lib.load().qssm_control_status_async(buf.ctl_ptr, buf.pinned.data_ptr(), stream))
 
 
@@ -319,6 +340,17 @@ def reset_workspaces() -> None:
 
 
 _plans: Dict[tuple, Plan] = {}
+_forward_keep = True
+
+
+def set_forward_keep(flag: bool) -> bool:
+    """Whether forwards planned from now on follow the planner's cache policy (`plan.keep_tiles`: the last tiles of
+    every chain load their operands with ordinary loads, for a backward that starts there) or stream every operand
+    past the caches (False).  Results are the same bit for bit; only what a launch leaves in the caches differs.
+    Returns the old setting."""
+    global _forward_keep
+    old, _forward_keep = _forward_keep, bool(flag)
+    return old
 
 
 def make_plan(B: int, L: int, D: int, in_dtype: torch.dtype, out_dtype: torch.dtype, direction: int,
@@ -432,14 +464,20 @@ def scan_forward(
 
     (x, a, b, c), strides, ptrs, align = _describe((x, a, b, c), (y, h), L, D)
 
+    keep = _forward_keep
+
     def make() -> _Launch:
         stride = 0
         if want_ckpt:
             # The backward decides how far apart the saved states may be; the forward follows.
             stride = make_plan(B, L, D, in_dtype, out_dtype, _lib.QSSM_BACKWARD, align, 0, bwd_tune).seg_len
-        return _Launch(make_plan(B, L, D, in_dtype, out_dtype, _lib.QSSM_FORWARD, align, stride, tune), ForwardCall())
+        plan = make_plan(B, L, D, in_dtype, out_dtype, _lib.QSSM_FORWARD, align, stride, tune)
+        if not keep:
+            plan = Plan.from_buffer_copy(plan)   # cached plans are shared: change a copy
+            plan.keep_tiles = 0
+        return _Launch(plan, ForwardCall())
 
-    entry = _launch_entry((0, B, L, D, in_dtype, out_dtype, align, want_ckpt, tune, bwd_tune), make)
+    entry = _launch_entry((0, B, L, D, in_dtype, out_dtype, align, want_ckpt, tune, bwd_tune, keep), make)
     ckpt = torch.empty((B, entry.n_ckpt, D), dtype=torch.float32, device=dev) if want_ckpt else None
 
     k = entry.call

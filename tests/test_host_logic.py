@@ -18,7 +18,7 @@ def test_library_exports_every_declared_symbol(hip_lib):
     assert declared == set(_lib.EXPORTED_SYMBOLS)
     for name in declared:
         assert getattr(hip_lib, name) is not None
-    assert hip_lib.qssm_version() == 100
+    assert hip_lib.qssm_version() == _lib.QSSM_VERSION == 200
     assert ctypes.sizeof(_lib.Plan) == 20 * 4 + 3 * 8
 
 
@@ -310,3 +310,92 @@ def test_tile_index_arithmetic_over_random_shapes(hip_lib):
             assert lo >= 0 and hi == B * L * D - 1, what
             assert hi_ckpt < plan.ckpt_elems, what
             assert hi_word <= plan.workspace_bytes, what
+
+
+class _FakeBuffers:
+    """What `_launch_buffers` and `_after_launch` touch of a `_Buffers` entry, without device or pinned memory."""
+
+    def __init__(self):
+        self.control = self.workspace = object()
+        self.ctl_ptr = self.ws_ptr = 256
+        self.ctl_size = self.ws_size = 1 << 30
+        self.epoch = 0
+        self.captured = False
+        self.seen = ctypes.c_int32(0)
+        self.since_check = 0
+        self.device = torch.device("cpu")
+        self.where = "a fake device"
+
+
+def test_launches_from_several_threads_get_distinct_numbers(monkeypatch):
+    # The caller's thread (next forward) and autograd's thread (a backward) may launch on one stream at the same
+    # time: two launches must never share a flag value, and every due status check must be asked for exactly once.
+    import sys
+    import threading
+
+    monkeypatch.setattr(torch._C, "_cuda_isCurrentStreamCapturing", lambda: False, raising=False)
+    asked = []
+    monkeypatch.setattr(hip_scan._lib, "load", lambda: type("L", (), {
+        "qssm_control_status_async": staticmethod(lambda *a: asked.append(1) or 0)})())
+    old_period = hip_scan.set_status_check_period(7)
+    key = (0, 0x1234, False)
+    buf = _FakeBuffers()
+    buf.pinned = type("P", (), {"data_ptr": staticmethod(lambda: 0)})()
+    hip_scan._buffers[key] = buf
+    n_threads, per_thread = 8, 4000
+    got = [[] for _ in range(n_threads)]
+    start = threading.Barrier(n_threads)
+    old_switch = sys.getswitchinterval()
+    sys.setswitchinterval(1e-6)   # hand the interpreter from thread to thread as often as it can
+
+    def work(slot):
+        start.wait()
+        for _ in range(per_thread):
+            b, epoch, capturing = hip_scan._launch_buffers(buf.device, 0, 0x1234, 64, 64)
+            got[slot].append(epoch)
+            hip_scan._after_launch(b, 0x1234, capturing)
+
+    try:
+        threads = [threading.Thread(target=work, args=(k,)) for k in range(n_threads)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+    finally:
+        sys.setswitchinterval(old_switch)
+        hip_scan.set_status_check_period(old_period)
+        hip_scan._buffers.pop(key, None)
+    flat = [e for part in got for e in part]
+    total = n_threads * per_thread
+    assert sorted(flat) == list(range(1, total + 1))
+    assert all(a < b for part in got for a, b in zip(part, part[1:]))   # and in order within a thread
+    assert len(asked) == total // 7 and buf.since_check == total % 7
+
+
+def test_device_side_launch_count_never_repeats_a_flag_between_wipes(hip_lib):
+    # Launches that number themselves (epoch argument 0) use flag count + 1 and the counting kernel stores the
+    # next count.  Walk the arithmetic across both wraps: no flag is ever zero, flags grow by one between restarts,
+    # and the static scratch array restarts its count only behind a launch whose prologue wiped it.
+    def step(count, static):
+        flag, nxt, wipes = ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_int32()
+        assert hip_lib.qssm_launch_count_step(count, static, ctypes.byref(flag), ctypes.byref(nxt), ctypes.byref(wipes)) == 0
+        return flag.value, nxt.value, wipes.value
+
+    for static, restart_from in ((1, 0xFFFFFFF0), (0, 0xFFFFFFFE)):
+        count, flags, wiped_at = restart_from - 3, [], []
+        for _ in range(8):
+            flag, nxt, wipes = step(count, static)
+            assert flag != 0 and flag == (count + 1) & 0xFFFFFFFF
+            if wipes:
+                wiped_at.append(count)
+            if nxt == 0:
+                # the count restarts: with the static array only behind a wipe, so flag 1 cannot meet an old word
+                assert count >= restart_from and (not static or wipes)
+            else:
+                assert nxt == count + 1
+            flags.append(flag)
+            count = nxt
+        assert flags[:4] == [restart_from - 2, restart_from - 1, restart_from, restart_from + 1]
+        assert flags[4:] == [1, 2, 3, 4]
+        assert wiped_at == ([0xFFFFFFF0] if static else [])
+    assert step(5, 1) == (6, 6, 0) and step(0, 0) == (1, 1, 0)
