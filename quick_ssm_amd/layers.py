@@ -35,6 +35,32 @@ class RMSNorm(nn.Module):
         return rms_norm(x, self.weight, self.eps)
 
 
+class _PackedProjection(torch.autograd.Function):
+    """u -> u @ wide_w^T + wide_b, where wide_w [5 S, H] and wide_b [5 S] are the memory of the five projection
+    weights and of A_proj's bias (`SSM._packed_parameters`).  The five weights and the bias are passed as well so
+    that autograd routes their gradients: one GEMM gives the gradient of the wide weight, whose row blocks go to the
+    five parameters; the bias gradient is summed over A_proj's block only."""
+
+    @staticmethod
+    def forward(ctx, u, w_a, w_b, w_ca, w_cb, w_d, bias_a, wide_w, wide_b):
+        ctx.save_for_backward(u, wide_w)
+        return torch.nn.functional.linear(u, wide_w, wide_b)
+
+    @staticmethod
+    def backward(ctx, g):
+        u, wide_w = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        S = wide_w.shape[0] // 5
+        g2 = g.reshape(-1, g.shape[-1])
+        du = (g2 @ wide_w).view_as(u) if need[0] else None
+        blocks = [None] * 5
+        if any(need[1:6]):
+            dw = g2.t() @ u.reshape(-1, u.shape[-1])                              # [5 S, H]
+            blocks = [dw[k * S:(k + 1) * S] if need[1 + k] else None for k in range(5)]
+        dbias = g2[:, :S].sum(0) if need[6] else None
+        return (du, *blocks, dbias, None, None)
+
+
 class SSM(nn.Module):
     """Gated linear recurrence layer: norm -> five projections -> scan -> out projection (+ residual)."""
 
@@ -71,24 +97,49 @@ class SSM(nn.Module):
     # Below this many elements per projection output a layer's step is bound by launches, not by their work.
     _BATCHED_PROJECTION_LIMIT = 1 << 23
 
+    def _packed_parameters(self):
+        """The five projection weights as one [5 S, H] tensor and a [5 S] bias (A_proj's, then zeros) that ARE the
+        parameters' memory: each `nn.Linear.weight` is a row block of the wide tensor, `A_proj.bias` the head of the
+        wide bias.  Parameter objects, names and values stay what they were (state dicts and optimizers see no
+        difference); only where their data lives changes, once.  Whatever gives the parameters storage of their own
+        again (`.to()`, `.half()`, loading into fresh tensors) is noticed here by their addresses and packed again."""
+        ws = (self.A_proj.weight, self.B_proj.weight, self.C_proj_a.weight, self.C_proj_b.weight, self.D_proj.weight)
+        S, H = self.state_size_dim, self.hidden_size
+        packed = self.__dict__.get("_packed")
+        if packed is not None:
+            wide_w, wide_b = packed
+            base, step = wide_w.data_ptr(), S * H * wide_w.element_size()
+            if (wide_w.dtype == ws[0].dtype and wide_b.dtype == self.A_proj.bias.dtype
+                    and all(w.data_ptr() == base + k * step for k, w in enumerate(ws))
+                    and self.A_proj.bias.data_ptr() == wide_b.data_ptr()):
+                return wide_w, wide_b
+        with torch.no_grad():
+            wide_w = torch.cat([w.data for w in ws])                              # [5 S, H]
+            for k, w in enumerate(ws):
+                w.data = wide_w[k * S:(k + 1) * S]
+            bias = self.A_proj.bias
+            wide_b = torch.cat((bias.data, bias.data.new_zeros(4 * S)))
+            bias.data = wide_b[:S]
+        self.__dict__["_packed"] = (wide_w, wide_b)
+        return wide_w, wide_b
+
     def _wide_projection(self, u: torch.Tensor) -> Optional[torch.Tensor]:
         """All five projection outputs as one [.., 5 S] tensor (blocks in A, B, C_a, C_b, D order) from a single GEMM
-        over the concatenated weights, for small layers; None for the others.
+        over the packed weights, for small layers; None for the others.
 
         The copy task's 12 x hidden 256 stack spends a training step on about a thousand launches of a few
-        microseconds each, 194 of them GEMMs: one GEMM forward and two backward per layer instead of five and ten
-        cut both the host's and the GPU's time (the wide tensor's blocks are read in place by the gate kernels, and
-        their gradients are written as blocks of one wide gradient).  The parameters stay the five separate
-        `nn.Linear` modules of the reference.  Large layers keep the separate GEMMs: theirs are efficient already,
-        and the bias gradient over the wide tensor would cost more than it saves."""
+        microseconds each: one GEMM forward and two backward per layer instead of five and ten cut both the host's
+        and the GPU's time (the wide tensor's blocks are read in place by the gate kernels, and their gradients are
+        written as blocks of one wide gradient).  The weights are not concatenated per call: the five parameters
+        live in one tensor (`_packed_parameters`), and the gradient of that tensor is handed back as five row blocks.
+        Large layers keep the separate GEMMs: theirs are efficient already."""
         S, H = self.state_size_dim, self.hidden_size
         rows = u.numel() // H
         if not (u.is_cuda and 0 < rows * S <= self._BATCHED_PROJECTION_LIMIT):
             return None
-        w = torch.cat((self.A_proj.weight, self.B_proj.weight, self.C_proj_a.weight, self.C_proj_b.weight,
-                       self.D_proj.weight))                                      # [5 S, H]
-        bias = torch.cat((self.A_proj.bias, self.A_proj.bias.new_zeros(4 * S)))
-        return torch.nn.functional.linear(u, w, bias)
+        wide_w, wide_b = self._packed_parameters()
+        return _PackedProjection.apply(u, self.A_proj.weight, self.B_proj.weight, self.C_proj_a.weight,
+                                       self.C_proj_b.weight, self.D_proj.weight, self.A_proj.bias, wide_w, wide_b)
 
     def gates(self, u: torch.Tensor):
         """The scan's four operands (x, a, b, c) from the normalised input, in `compute_dtype`."""

@@ -399,3 +399,54 @@ def test_device_side_launch_count_never_repeats_a_flag_between_wipes(hip_lib):
         assert flags[4:] == [1, 2, 3, 4]
         assert wiped_at == ([0xFFFFFFF0] if static else [])
     assert step(5, 1) == (6, 6, 0) and step(0, 0) == (1, 1, 0)
+
+
+def test_packed_projection_parameters_stay_the_reference_parameters():
+    # Small layers run one GEMM over the five projection weights, which then live in one [5 S, H] tensor.  Names,
+    # values and Parameter objects stay the reference's; optimizer updates and state-dict loads keep the packing;
+    # whatever moves the parameters to storage of their own is noticed and packed again; and the packed function
+    # gives the values and gradients of the five separate nn.Linear calls.
+    import copy
+
+    from quick_ssm_amd.layers import SSM, _PackedProjection
+
+    torch.manual_seed(0)
+    layer = SSM(16, 2.0, compute_dtype=torch.float32)
+    S, H = 32, 16
+    before = {k: v.clone() for k, v in layer.state_dict().items()}
+    params = dict(layer.named_parameters())
+    wide_w, wide_b = layer._packed_parameters()
+    assert wide_w.shape == (5 * S, H) and wide_b.shape == (5 * S,)
+    assert dict(layer.named_parameters()).keys() == params.keys()
+    assert all(p is params[n] for n, p in layer.named_parameters())
+    for k, v in layer.state_dict().items():
+        assert torch.equal(v, before[k]), k
+    order = ("A_proj", "B_proj", "C_proj_a", "C_proj_b", "D_proj")
+    for k, n in enumerate(order):
+        assert getattr(layer, n).weight.data_ptr() == wide_w.data_ptr() + k * S * H * 4
+    opt = torch.optim.AdamW(layer.parameters(), lr=0.1)
+    for p in layer.parameters():
+        p.grad = torch.ones_like(p)
+    opt.step()
+    again_w, again_b = layer._packed_parameters()
+    assert again_w is wide_w and again_b is wide_b                       # in-place updates keep the packing
+    assert torch.equal(wide_w[S:2 * S], layer.B_proj.weight) and not torch.equal(layer.B_proj.weight, before["B_proj.weight"])
+    assert torch.equal(wide_b[:S], layer.A_proj.bias) and float(wide_b[S:].abs().max()) == 0.0
+    twin = copy.deepcopy(layer)
+    twin_w, _ = twin._packed_parameters()
+    assert twin_w.data_ptr() != wide_w.data_ptr() and twin.A_proj.weight.data_ptr() == twin_w.data_ptr()
+    layer.double()                                                       # new storage per parameter: packed again
+    new_w, _ = layer._packed_parameters()
+    assert new_w.dtype == torch.float64 and layer.D_proj.weight.data_ptr() == new_w.data_ptr() + 4 * S * H * 8
+    layer.load_state_dict({k: v.double() for k, v in before.items()})
+    kept_w, _ = layer._packed_parameters()
+    assert kept_w is new_w and torch.equal(kept_w[S:2 * S].float(), before["B_proj.weight"])
+
+    u = torch.randn(3, 5, H, dtype=torch.double, requires_grad=True)
+    out = _PackedProjection.apply(u, *(getattr(layer, n).weight for n in order), layer.A_proj.bias, *layer._packed_parameters())
+    ref = torch.cat([getattr(layer, n)(u) for n in order], dim=-1)
+    assert torch.allclose(out, ref, rtol=1e-12, atol=1e-12)
+    wrt = [u] + [getattr(layer, n).weight for n in order] + [layer.A_proj.bias]
+    g = torch.randn_like(out)
+    for got, want in zip(torch.autograd.grad(out, wrt, g), torch.autograd.grad(ref, wrt, g)):
+        assert torch.allclose(got, want, rtol=1e-12, atol=1e-12)
