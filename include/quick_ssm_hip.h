@@ -87,6 +87,9 @@ typedef struct qssm_plan {
   int32_t keep_tiles;     /* forward: the last keep_tiles tiles of every chain load their operands with ordinary
                              loads, so that the backward, which starts there, finds them in the caches; the rest
                              streams past the caches.  0 switches it off. */
+  int32_t compute_dtype;  /* gated scans: the type the layer rounds its gates' outputs to (its compute dtype): the
+                             projections' storage type, or QSSM_F16 / QSSM_BF16 for fp32 projections.  Plain scans:
+                             in_dtype. */
   uint64_t control_bytes;   /* control block the launch needs (status word + ticket counters) */
   uint64_t workspace_bytes; /* workspace the launch needs (words exchanged between workgroups) */
   uint64_t ckpt_elems;      /* B * n_ckpt * D floats */
@@ -386,15 +389,21 @@ QSSM_API int qssm_gates_backward_strided(const void* g_a, const void* g_x, const
  * s = sigmoid(Ca), with da, db, dc rounded to the storage type as qssm_scan_backward stores them.  The tensors a,
  * x, b, c and their gradients never reach HBM: 12 instead of 30 bytes per element forward and 22 instead of 46
  * backward for bf16.
- *   - Plans come from qssm_plan_scan_gated (one geometry: 4 columns x 8 steps per lane, 256 lanes); shapes it
- *     refuses (D < 128, rows not 16-byte aligned, fp32 projections) take qssm_gates_* + qssm_scan_*.
+ *   - fp32 projections (the reference's default layer: fp32 parameters, 16-bit compute dtype) are taken as well:
+ *     `compute_dtype` then names the 16-bit type (or QSSM_F32) the gates' outputs and the scan's gradients are
+ *     rounded to, in registers, where the layer's casts round them; y and dy are f32.  20 + 4 instead of 28 + 12
+ *     bytes per element forward, 24 + 20 instead of 44 + 20 backward.
+ *   - Plans come from qssm_plan_scan_gated (one geometry: 8 bytes x 8 steps per lane, 256 lanes); shapes it
+ *     refuses (D < 128, rows not 16-byte aligned) take qssm_gates_* + qssm_scan_*.
  *   - ckpt, control, workspace, epoch: as for qssm_scan_forward / qssm_scan_backward; the backward needs the saved
- *     states (the checkpoint=True case) and y / dy stored as the projections are (forward: or as f32).
+ *     states (the checkpoint=True case) and y / dy stored as the projections are (16-bit projections forward: or
+ *     as f32).
  * Replaces SSM.forward's elementwise chain and scan call, quick_ssm/layers.py:76-104, and what autograd records
  * for them.
  */
-QSSM_API int qssm_plan_scan_gated(int32_t B, int32_t L, int32_t D, int32_t dtype, int32_t out_dtype,
-                         int32_t direction, int32_t align_elems, int32_t ckpt_stride, qssm_plan* plan);
+QSSM_API int qssm_plan_scan_gated(int32_t B, int32_t L, int32_t D, int32_t dtype, int32_t compute_dtype,
+                         int32_t out_dtype, int32_t direction, int32_t align_elems, int32_t ckpt_stride,
+                         qssm_plan* plan);
 
 QSSM_API int qssm_scan_gated_forward(const qssm_plan* plan,
                             const void* A_pre, qssm_strides sA,

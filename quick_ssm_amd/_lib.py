@@ -74,6 +74,7 @@ class Plan(ctypes.Structure):
         ("n_ckpt", ctypes.c_int32),
         ("lds_bytes", ctypes.c_int32),
         ("keep_tiles", ctypes.c_int32),
+        ("compute_dtype", ctypes.c_int32),
         ("control_bytes", ctypes.c_uint64),
         ("workspace_bytes", ctypes.c_uint64),
         ("ckpt_elems", ctypes.c_uint64),
@@ -166,7 +167,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         + [vp, u64, vp, u64, ctypes.c_uint32, vp]
     )
     lib.qssm_plan_scan_gated.restype = ctypes.c_int
-    lib.qssm_plan_scan_gated.argtypes = [i32] * 8 + [ctypes.POINTER(Plan)]
+    lib.qssm_plan_scan_gated.argtypes = [i32] * 9 + [ctypes.POINTER(Plan)]
     lib.qssm_scan_gated_forward.restype = ctypes.c_int
     lib.qssm_scan_gated_forward.argtypes = (
         [ctypes.POINTER(Plan)] + [vp, Strides] * 6 + [vp] + [vp, u64, vp, u64, ctypes.c_uint32, vp]

@@ -184,6 +184,11 @@ struct GateExtras {
   qssm_strides sdc2;
 };
 
+// What a launch tells its kernel table about gating: the plan's compute dtype for a gated launch.
+static int gated_code(const qssm_plan* plan, const GateExtras* gate) {
+  return gate == nullptr ? kNotGated : plan->compute_dtype;
+}
+
 static int forward_launch(const qssm_plan* plan, const void* x, qssm_strides sx, const void* a, qssm_strides sa,
                           const void* b, qssm_strides sb, const void* c, qssm_strides sc, void* y, qssm_strides sy,
                           float* h_out, qssm_strides sh, float* ckpt, const float* h_init, float* h_final,
@@ -211,13 +216,21 @@ int qssm_plan_scan(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int32_t ou
 // The gated kernels exist in one shape: 4 columns (8 bytes of 16-bit storage) and 8 steps per lane, 256 lanes,
 // rows of 64 or 32 lanes, clusters of at most two tiles (the backward's three LDS-resident operands leave LDS
 // for no more neighbour maps).
-static const int32_t kGatedTune = (8 << 8) | (4 << 16) | (1 << 24);
-int qssm_plan_scan_gated(int32_t B, int32_t L, int32_t D, int32_t dtype, int32_t out_dtype, int32_t direction,
-                         int32_t align_elems, int32_t ckpt_stride, qssm_plan* plan) {
-  if (dtype_size(dtype) != 2) return fail(QSSM_EINVAL, "the gated scan is built for 16-bit projections");
-  if (D % 4 != 0 || align_elems % 8 != 0 || D < 128)
+int qssm_plan_scan_gated(int32_t B, int32_t L, int32_t D, int32_t dtype, int32_t compute_dtype, int32_t out_dtype,
+                         int32_t direction, int32_t align_elems, int32_t ckpt_stride, qssm_plan* plan) {
+  const int es = dtype_size(dtype);
+  if (es == 0 || dtype_size(compute_dtype) == 0) return fail(QSSM_EINVAL, "unknown dtype code");
+  if (es == 2 && compute_dtype != dtype)
+    return fail(QSSM_EINVAL, "16-bit projections are their own compute dtype");
+  if (es == 4 && out_dtype != QSSM_F32)
+    return fail(QSSM_EINVAL, "the gated scan over fp32 projections stores y and dy as fp32");
+  // 8 bytes per lane and 8 steps per lane, 256 lanes: 4 columns of 16-bit storage, 2 of fp32
+  const int vec = 8 / es;
+  if (D % 4 != 0 || (align_elems * es) % 16 != 0 || D < 128)
     return fail(QSSM_EALIGN, "the gated scan needs D >= 128, a multiple of 4, and 16-byte aligned rows");
+  const int32_t kGatedTune = (8 << 8) | (vec << 16) | (1 << 24);
   int rc = qssm_plan_scan_tuned(B, L, D, dtype, out_dtype, direction, align_elems, ckpt_stride, kGatedTune, plan);
+  if (rc == 0) plan->compute_dtype = compute_dtype;
   if (rc != 0 || B == 0 || L == 0) return rc;
   int g_log2 = plan->g_log2 > 6 ? 6 : (plan->g_log2 < 5 ? 5 : plan->g_log2);
   if (g_log2 != plan->g_log2)
@@ -227,7 +240,8 @@ int qssm_plan_scan_gated(int32_t B, int32_t L, int32_t D, int32_t dtype, int32_t
     rc = qssm_plan_scan_tuned(B, L, D, dtype, out_dtype, direction, align_elems, ckpt_stride,
                               kGatedTune | (g_log2 + 1) | (2 << 28), plan);
   if (rc != 0) return rc;
-  if (plan->vec != 4 || plan->steps != 8 || plan->threads != 256 || (plan->g_log2 != 6 && plan->g_log2 != 5) ||
+  plan->compute_dtype = compute_dtype;
+  if (plan->vec != vec || plan->steps != 8 || plan->threads != 256 || (plan->g_log2 != 6 && plan->g_log2 != 5) ||
       plan->cluster > 2)
     return fail(QSSM_EINVAL, "no gated geometry for this shape");
   return 0;
@@ -251,6 +265,7 @@ int qssm_plan_scan_tuned(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int3
   plan->D = D;
   plan->in_dtype = in_dtype;
   plan->out_dtype = out_dtype;
+  plan->compute_dtype = in_dtype;
   plan->direction = direction;
 
   // Widest lane vector the alignment allows: 8 bytes per lane for 16-bit storage, 16 for fp32
@@ -540,13 +555,16 @@ static int forward_launch(const qssm_plan* plan, const void* x, qssm_strides sx,
   // c can live in LDS instead of registers when a row of the strip is one wavefront of 8-byte lanes
   // and c's rows can be fetched 16 bytes at a time.
   size_t lds = (size_t)plan->lds_bytes;
-  const bool narrow_rows = v == 4 && (plan->g_log2 == 6 || plan->g_log2 == 5) && (plan->threads == 256 || plan->threads == 512);
-  const bool wide_rows = v == 8 && (plan->threads == 256 || plan->threads == 512);   // every lane fetches its own 16 bytes
-  bool c_in_lds = y != nullptr && c != nullptr && es == 2 && ((narrow_rows && plan->steps == 8) || wide_rows) &&
+  // (8 bytes per lane: 4 columns of 16-bit storage; 2 columns of fp32 only in the gated scan's kernels)
+  const bool narrow_rows = v * es == 8 && (es == 2 || gate != nullptr) && (plan->g_log2 == 6 || plan->g_log2 == 5) &&
+                           (plan->threads == 256 || plan->threads == 512);
+  const bool wide_rows = es == 2 && v == 8 && (plan->threads == 256 || plan->threads == 512);   // every lane fetches its own 16 bytes
+  bool c_in_lds = y != nullptr && c != nullptr && ((narrow_rows && plan->steps == 8) || wide_rows) &&
                   ((uintptr_t)c) % 16 == 0 && (sc.b * es) % 16 == 0 && (sc.l * es) % 16 == 0 &&
                   lds + fwd_c_lds_bytes(plan->threads, plan->steps, v * es) <= (size_t)kMaxLdsBytes;
   if (c_in_lds) lds += fwd_c_lds_bytes(plan->threads, plan->steps, v * es);
   args.c2 = nullptr; args.c2_sb = args.c2_sl = 0;
+  if (gate != nullptr && dtype_size(plan->compute_dtype) == 0) return fail(QSSM_EINVAL, "plan.compute_dtype is not a dtype code");
   if (gate != nullptr) {
     // Ca and Cb both go through LDS: the same conditions again for Cb, and room for the second array
     if (!c_in_lds || !narrow_rows || plan->threads != 256 || gate->c2 == nullptr || ((uintptr_t)gate->c2) % 16 != 0 ||
@@ -556,7 +574,7 @@ static int forward_launch(const qssm_plan* plan, const void* x, qssm_strides sx,
     lds += fwd_c_lds_bytes(plan->threads, plan->steps, v * es);
     args.c2 = gate->c2; args.c2_sb = gate->sc2.b; args.c2_sl = gate->sc2.l;
   }
-  if (!fn(args, plan->vec, plan->steps, plan->threads, c_in_lds, gate != nullptr, grid, lds, (hipStream_t)stream))
+  if (!fn(args, plan->vec, plan->steps, plan->threads, c_in_lds, gated_code(plan, gate), grid, lds, (hipStream_t)stream))
     return fail(QSSM_EINVAL, "no forward kernel for vec=%d steps=%d threads=%d", plan->vec, plan->steps, plan->threads);
   if (epoch == 0 && plan->n_seg > 1)
     hipLaunchKernelGGL(count_launch_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream,
@@ -644,12 +662,15 @@ static int backward_launch(const qssm_plan* plan, const void* x, qssm_strides sx
   // c and dy can live in LDS instead of registers when a row of the strip is one wavefront of 8-byte
   // lanes in both and their rows can be fetched 16 bytes at a time.
   size_t lds = (size_t)plan->lds_bytes;
-  bool cg_in_lds = es == 2 && (os == 2 || os == 4) && v == 4 && (plan->g_log2 == 6 || plan->g_log2 == 5) && plan->steps == 8 && plan->threads == 256 &&
+  // (8 bytes per lane: 4 columns of 16-bit storage; 2 columns of fp32, with fp32 dy, only in the gated scan's kernels)
+  bool cg_in_lds = ((es == 2 && (os == 2 || os == 4) && v == 4) || (gate != nullptr && es == 4 && os == 4 && v == 2)) &&
+                   (plan->g_log2 == 6 || plan->g_log2 == 5) && plan->steps == 8 && plan->threads == 256 &&
                    ((uintptr_t)c) % 16 == 0 && (sc.b * es) % 16 == 0 && (sc.l * es) % 16 == 0 &&
                    ((uintptr_t)dy) % 16 == 0 && (sdy.b * os) % 16 == 0 && (sdy.l * os) % 16 == 0 &&
                    lds + bwd_cg_lds_bytes(plan->threads, plan->steps) <= (size_t)kMaxLdsBytes;
   if (cg_in_lds) lds += bwd_cg_lds_bytes(plan->threads, plan->steps);
   args.c2 = nullptr; args.c2_sb = args.c2_sl = 0; args.dc2 = nullptr; args.dc2_sb = args.dc2_sl = 0;
+  if (gate != nullptr && dtype_size(plan->compute_dtype) == 0) return fail(QSSM_EINVAL, "plan.compute_dtype is not a dtype code");
   if (gate != nullptr) {
     // Ca, Cb and dy all go through LDS: the same conditions again for Cb, and room for the third array
     const size_t one = bwd_cg_lds_bytes(plan->threads, plan->steps) / 2;
@@ -657,13 +678,13 @@ static int backward_launch(const qssm_plan* plan, const void* x, qssm_strides sx
         (gate->sc2.l * es) % 16 != 0 || !tile_span_ok(plan, gate->c2, gate->sc2.b, gate->sc2.l, es) ||
         !aligned_to(gate->dc2, gate->sdc2.b, gate->sdc2.l, es, v) || !tile_span_ok(plan, gate->dc2, gate->sdc2.b, gate->sdc2.l, es) ||
         lds + one > (size_t)kMaxLdsBytes)
-      return fail(QSSM_EALIGN, "gated scan needs a plan of qssm_plan_scan_gated, 16-bit dy, saved states, and Ca, Cb, dy with "
-                               "16-byte aligned rows");
+      return fail(QSSM_EALIGN, "gated scan needs a plan of qssm_plan_scan_gated, dy stored as the projections are, saved "
+                               "states, and Ca, Cb, dy with 16-byte aligned rows");
     lds += one;
     args.c2 = gate->c2; args.c2_sb = gate->sc2.b; args.c2_sl = gate->sc2.l;
     args.dc2 = gate->dc2; args.dc2_sb = gate->sdc2.b; args.dc2_sl = gate->sdc2.l;
   }
-  if (!fn(args, plan->vec, plan->steps, plan->threads, cg_in_lds, gate != nullptr, grid, lds, (hipStream_t)stream))
+  if (!fn(args, plan->vec, plan->steps, plan->threads, cg_in_lds, gated_code(plan, gate), grid, lds, (hipStream_t)stream))
     return fail(QSSM_EINVAL, "no backward kernel for vec=%d steps=%d threads=%d", plan->vec, plan->steps, plan->threads);
   if (epoch == 0 && plan->n_seg > 1)
     hipLaunchKernelGGL(count_launch_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream,

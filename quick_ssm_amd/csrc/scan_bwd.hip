@@ -16,6 +16,8 @@
 // has to be fetched across a tile edge (the reference kernel loads the shifted a,
 // triton_backwards.py:62-66).  Over a run of steps the map E_in -> E_out is affine with the same
 // multiplier prod a(t) as the forward map, so one product serves both directions.
+#include <type_traits>
+
 #include "scan_common.h"
 
 namespace qssm {
@@ -39,13 +41,18 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 //
 // XLANE: rows of 16 lanes or fewer (a few columns of D), where a tile has 16 to 256 lane groups: their maps are
 // combined, in both directions, by exchanges between the lanes of a wavefront instead of two walks through LDS.
-template <typename Tin, typename Tout, int VEC, int T, int NTH, bool CLDS, bool GATED, bool XLANE>
+//
+// Tc is the type the layer rounds the gates' outputs and the scan's gradients to (its compute dtype): the projections'
+// storage type, or a 16-bit type that only exists in registers when the projections are fp32.
+template <typename Tin, typename Tout, int VEC, int T, int NTH, bool CLDS, bool GATED, bool XLANE, typename Tc = Tin>
 __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
   static_assert(!GATED || CLDS, "gated scan: Ca, Cb and dy through LDS");
+  static_assert(GATED || std::is_same<Tc, Tin>::value, "a compute dtype of its own only means something to the gated scan");
+  constexpr bool ROUND = !std::is_same<Tc, Tin>::value;   // gate outputs and scan gradients are rounded to a type narrower than their storage
   static_assert(!XLANE || (!CLDS && !GATED), "cross-lane fold: register-only operands");
   static_assert(!CLDS || (sizeof(Tin) * VEC == 8 && (sizeof(Tout) * VEC == 8 || sizeof(Tout) * VEC == 16) && T % 2 == 0),
                 "LDS-resident c and dy: 8 bytes per lane (dy alone: 16), even step count");
-  static_assert(!GATED || sizeof(Tout) * VEC == 8, "gated scan: 16-bit dy");
+  static_assert(!GATED || sizeof(Tout) * VEC == 8, "gated scan: dy at 8 bytes per lane");
   constexpr bool GW = CLDS && sizeof(Tout) * VEC == 16;   // dy alone in LDS, 16 bytes per lane
   constexpr bool CREG = !CLDS || GW;                       // c in registers
   extern __shared__ __align__(16) float lds[];
@@ -348,6 +355,15 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
           fa[v] = ga[v] * (1.0f - ga[v]);
           fb[v] = gb[v] * (1.0f - gb[v]);
         }
+        if constexpr (ROUND) {
+          float gx[VEC];
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) gx[v] = elem(rx[i], v);
+          round_through<Tc, VEC>(ga);
+          round_through<Tc, VEC>(gb);
+          round_through<Tc, VEC>(gx);
+          ElemBits<Tin>::template set<VEC>(rx[i], gx);
+        }
         ElemBits<Tin>::template set<VEC>(ra[i], ga);
         ElemBits<Tin>::template set<VEC>(rb[i], gb);
         ElemBits<Tin>::template set<VEC>(za[i], fa);
@@ -378,6 +394,7 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
       float gc[VEC];
 #pragma unroll
       for (int v = 0; v < VEC; ++v) { const float ca = elem(cw, v); gc[v] = ca * sigmoid_f(ca) * elem(cw2, v); }
+      if constexpr (ROUND) round_through<Tc, VEC>(gc);
       ElemBits<Tin>::template set<VEC>(cw, gc);
     }
 #pragma unroll
@@ -628,6 +645,7 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
         sg[v] = sigmoid_f(zca[v]);
         gc[v] = zca[v] * sg[v] * zcb[v];
       }
+      if constexpr (ROUND) round_through<Tc, VEC>(gc);
       ElemBits<Tin>::template set<VEC>(cw, gc);
     }
 #pragma unroll
@@ -643,9 +661,10 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
     }
     if constexpr (GATED) {
       // the scan's gradients as it would have stored them, then through the activations' derivatives
-      round_through<Tin, VEC>(vda);
-      round_through<Tin, VEC>(vdb);
-      round_through<Tin, VEC>(vdc);
+      if constexpr (ROUND) round_through<Tc, VEC>(vdx);   // (stored as Tin below: the same rounding when Tc is Tin)
+      round_through<Tc, VEC>(vda);
+      round_through<Tc, VEC>(vdb);
+      round_through<Tc, VEC>(vdc);
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
         vda[v] = vda[v] * elem(za[i], v);
@@ -676,12 +695,23 @@ __global__ void __launch_bounds__(NTH) scan_bwd_kernel(const BwdArgs p) {
 }
 
 template <typename Tin, typename Tout>
-static bool launch_bwd(const BwdArgs& args, int vec, int steps, int threads, bool cg_in_lds, bool gated, dim3 grid,
+static bool launch_bwd(const BwdArgs& args, int vec, int steps, int threads, bool cg_in_lds, int gated, dim3 grid,
                        size_t lds, hipStream_t stream) {
-  if (gated) {
+  if (gated != kNotGated) {
+    // `gated` names the layer's compute dtype: the projections' storage type itself, or a 16-bit type for fp32 ones
     if constexpr (sizeof(Tin) == 2 && sizeof(Tout) == 2) {
-      if (vec == 4 && steps == 8 && threads == 256 && cg_in_lds) {
+      if (vec == 4 && steps == 8 && threads == 256 && cg_in_lds && gated == dtype_code<Tin>()) {
         hipLaunchKernelGGL((scan_bwd_kernel<Tin, Tout, 4, 8, 256, true, true, false>), grid, dim3(256), lds, stream, args);
+        return true;
+      }
+    } else if constexpr (sizeof(Tin) == 4 && sizeof(Tout) == 4) {
+      if (vec == 2 && steps == 8 && threads == 256 && cg_in_lds) {
+        if (gated == QSSM_F32)
+          hipLaunchKernelGGL((scan_bwd_kernel<float, float, 2, 8, 256, true, true, false, float>), grid, dim3(256), lds, stream, args);
+        else if (gated == QSSM_F16)
+          hipLaunchKernelGGL((scan_bwd_kernel<float, float, 2, 8, 256, true, true, false, f16_t>), grid, dim3(256), lds, stream, args);
+        else
+          hipLaunchKernelGGL((scan_bwd_kernel<float, float, 2, 8, 256, true, true, false, bf16_t>), grid, dim3(256), lds, stream, args);
         return true;
       }
     }

@@ -479,11 +479,17 @@ inline size_t bwd_lds_bytes(int nth, int vec, int cols, int cluster) {
 
 // Host-side launch tables, one entry per (in dtype, out dtype) pair the library instantiates.
 // Return false if (vec, steps, threads) is not an instantiated combination.
-typedef bool (*fwd_launch_fn)(const FwdArgs&, int vec, int steps, int threads, bool c_in_lds, bool gated, dim3 grid,
+// `gated`: kNotGated for the plain scan, else the storage code of the layer's compute dtype (gated scan).
+constexpr int kNotGated = -1;
+template <typename T> constexpr int dtype_code();
+template <> constexpr int dtype_code<float>() { return QSSM_F32; }
+template <> constexpr int dtype_code<f16_t>() { return QSSM_F16; }
+template <> constexpr int dtype_code<bf16_t>() { return QSSM_BF16; }
+typedef bool (*fwd_launch_fn)(const FwdArgs&, int vec, int steps, int threads, bool c_in_lds, int gated, dim3 grid,
                               size_t lds, hipStream_t stream);
 // Extra dynamic LDS of the forward kernel that keeps c in LDS: 8 or 16 bytes per lane and step.
 inline size_t fwd_c_lds_bytes(int nth, int steps, int lane_bytes) { return (size_t)nth * steps * lane_bytes; }
-typedef bool (*bwd_launch_fn)(const BwdArgs&, int vec, int steps, int threads, bool cg_in_lds, bool gated, dim3 grid,
+typedef bool (*bwd_launch_fn)(const BwdArgs&, int vec, int steps, int threads, bool cg_in_lds, int gated, dim3 grid,
                               size_t lds, hipStream_t stream);
 // Extra dynamic LDS of the backward kernel that keeps c and dy in LDS.
 inline size_t bwd_cg_lds_bytes(int nth, int steps) { return (size_t)2 * nth * steps * 8; }

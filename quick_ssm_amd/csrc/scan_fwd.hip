@@ -26,12 +26,18 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // compute dtype rounds them), c = silu(Ca) * Cb is formed step by step in the last sweep from two LDS-resident
 // operands.  The a, x, b, c tensors of the layer never exist in HBM.
 //
+// Tc is the type the layer rounds the gates' outputs to (its compute dtype): the projections' own storage type, or,
+// for fp32 projections (the reference's default layer: fp32 parameters, fp16 compute), a 16-bit type that only
+// ever exists in registers; a = sigmoid(A_pre), x = B_in, b and c are rounded through it before they are used.
+//
 // XLANE: rows of 16 lanes or fewer (a few columns of D), where a tile has 16 to 256 lane groups: their maps are
 // combined by exchanges between the lanes of a wavefront instead of a walk through LDS.
-template <typename Tin, typename Tout, int VEC, int T, int NTH, bool CLDS, bool GATED, bool XLANE>
+template <typename Tin, typename Tout, int VEC, int T, int NTH, bool CLDS, bool GATED, bool XLANE, typename Tc = Tin>
 __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
   static_assert(!XLANE || (!CLDS && !GATED), "cross-lane fold: register-only operands");
-  static_assert(!GATED || (CLDS && sizeof(Tin) * VEC == 8), "gated scan: 16-bit projections, Ca and Cb through LDS");
+  static_assert(!GATED || (CLDS && sizeof(Tin) * VEC == 8), "gated scan: 8 bytes per lane, Ca and Cb through LDS");
+  static_assert(GATED || std::is_same<Tc, Tin>::value, "a compute dtype of its own only means something to the gated scan");
+  constexpr bool ROUND = !std::is_same<Tc, Tin>::value;   // the gates' outputs are rounded to a type narrower than their storage
   static_assert(!CLDS || ((sizeof(Tin) * VEC == 8 || sizeof(Tin) * VEC == 16) && T % 2 == 0),
                 "LDS-resident c: 8 or 16 bytes per lane, even step count");
   // 16 bytes per lane: the load that deposits c in LDS gives every lane exactly its own columns of one step.
@@ -279,6 +285,15 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
         float ga[VEC], gb[VEC];
 #pragma unroll
         for (int v = 0; v < VEC; ++v) { ga[v] = sigmoid_f(elem(ra[i], v)); gb[v] = sigmoid_f(elem(rb[i], v)); }
+        if constexpr (ROUND) {
+          float gx[VEC];
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) gx[v] = elem(rx[i], v);
+          round_through<Tc, VEC>(ga);
+          round_through<Tc, VEC>(gb);
+          round_through<Tc, VEC>(gx);
+          ElemBits<Tin>::template set<VEC>(rx[i], gx);
+        }
         ElemBits<Tin>::template set<VEC>(ra[i], ga);
         ElemBits<Tin>::template set<VEC>(rb[i], gb);
       }
@@ -479,6 +494,7 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
       float gc[VEC];
 #pragma unroll
       for (int v = 0; v < VEC; ++v) { const float ca = elem(cw, v); gc[v] = ca * sigmoid_f(ca) * elem(cw2, v); }
+      if constexpr (ROUND) round_through<Tc, VEC>(gc);
       ElemBits<Tin>::template set<VEC>(cw, gc);
     }
 #pragma unroll
@@ -504,12 +520,23 @@ __global__ void __launch_bounds__(NTH) scan_fwd_kernel(const FwdArgs p) {
 }
 
 template <typename Tin, typename Tout>
-static bool launch_fwd(const FwdArgs& args, int vec, int steps, int threads, bool c_in_lds, bool gated, dim3 grid,
+static bool launch_fwd(const FwdArgs& args, int vec, int steps, int threads, bool c_in_lds, int gated, dim3 grid,
                        size_t lds, hipStream_t stream) {
-  if (gated) {
+  if (gated != kNotGated) {
+    // `gated` names the layer's compute dtype: the projections' storage type itself, or a 16-bit type for fp32 ones
     if constexpr (sizeof(Tin) == 2) {
-      if (vec == 4 && steps == 8 && threads == 256 && c_in_lds) {
+      if (vec == 4 && steps == 8 && threads == 256 && c_in_lds && gated == dtype_code<Tin>()) {
         hipLaunchKernelGGL((scan_fwd_kernel<Tin, Tout, 4, 8, 256, true, true, false>), grid, dim3(256), lds, stream, args);
+        return true;
+      }
+    } else if constexpr (sizeof(Tout) == 4) {
+      if (vec == 2 && steps == 8 && threads == 256 && c_in_lds) {
+        if (gated == QSSM_F32)
+          hipLaunchKernelGGL((scan_fwd_kernel<float, float, 2, 8, 256, true, true, false, float>), grid, dim3(256), lds, stream, args);
+        else if (gated == QSSM_F16)
+          hipLaunchKernelGGL((scan_fwd_kernel<float, float, 2, 8, 256, true, true, false, f16_t>), grid, dim3(256), lds, stream, args);
+        else
+          hipLaunchKernelGGL((scan_fwd_kernel<float, float, 2, 8, 256, true, true, false, bf16_t>), grid, dim3(256), lds, stream, args);
         return true;
       }
     }

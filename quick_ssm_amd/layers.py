@@ -171,7 +171,8 @@ class SSM(nn.Module):
         w_dtype = self.out_proj.weight.dtype
         out_dtype = w_dtype if scan_out_dtype is None else scan_out_dtype
         if backend in ("auto", "hip", "triton") and u.is_cuda and not _scan_interface._HONOR_TILES:
-            # 16-bit projections stored as the compute dtype: the activations happen inside the scan's launches
+            # 16-bit projections stored as the compute dtype, or fp32 projections with fp32 y: the activations (and the
+            # casts to the compute dtype) happen inside the scan's launches
             wide = self._wide_projection(u)
             if wide is not None:
                 S = self.state_size_dim
@@ -179,9 +180,9 @@ class SSM(nn.Module):
             else:
                 pre = (self.A_proj(u), self.B_proj(u), self.C_proj_a(u), self.C_proj_b(u), self.D_proj(u))
             if wide is not None and wide.dim() == 3 and _gated.supported(pre, self.compute_dtype, out_dtype, checkpoint):
-                y = _gated.gated_scan_wide(wide, out_dtype=out_dtype)
+                y = _gated.gated_scan_wide(wide, out_dtype=out_dtype, compute_dtype=self.compute_dtype)
             elif _gated.supported(pre, self.compute_dtype, out_dtype, checkpoint):
-                y = _gated.gated_scan(*pre, out_dtype=out_dtype)
+                y = _gated.gated_scan(*pre, out_dtype=out_dtype, compute_dtype=self.compute_dtype)
             else:
                 if wide is not None:
                     forget, drive, out_gate, in_gate = gate_prologue_wide(wide, self.compute_dtype)

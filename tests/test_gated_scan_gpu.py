@@ -44,10 +44,11 @@ def _oracle(pre, dy, dtype):
     return y, grads
 
 
-def _run(pre, dy, gpu, out_dtype, place=lambda t, dev: t.to(dev)):
+def _run(pre, dy, gpu, out_dtype, place=lambda t, dev: t.to(dev), compute_dtype=None):
     leaves = [place(t, gpu).detach().requires_grad_(True) for t in pre]
-    assert gated_scan.supported(leaves, pre[0].dtype, out_dtype)
-    y = gated_scan.gated_scan(*leaves, out_dtype=out_dtype)
+    compute_dtype = compute_dtype or pre[0].dtype
+    assert gated_scan.supported(leaves, compute_dtype, out_dtype)
+    y = gated_scan.gated_scan(*leaves, out_dtype=out_dtype, compute_dtype=compute_dtype)
     y.backward(place(dy, gpu))
     assert hip_scan.workspace_status() == 0
     return y.detach().cpu(), [t.grad.cpu() for t in leaves]
@@ -66,6 +67,64 @@ def test_gated_scan_matches_oracle_composition(gpu, dtype, shape):
     for name, got, want in zip(NAMES, grads, g_ref):
         assert got.dtype == dtype
         assert_close(name, got, want, TOL[dtype])
+
+
+@pytest.mark.parametrize("compute", [torch.float16, torch.bfloat16, torch.float32], ids=["c16", "cbf16", "c32"])
+@pytest.mark.parametrize("shape", [(2, 700, 512), (2, 1100, 264), (1, 97, 256), (3, 33, 128), (1, 2100, 136), (4, 2048, 1024)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_gated_scan_over_fp32_projections_matches_oracle_composition(gpu, compute, shape):
+    # The reference's default layer: fp32 projection outputs, gates and scan operands cast to the compute dtype
+    # (quick_ssm/layers.py:85-88), fp32 y and dy.  One launch each way; the 16-bit operands exist in registers only.
+    # Oracle: float64 gates, operands rounded to the compute dtype, float64 scan, float64 gate derivatives.
+    pre = _projections(shape, torch.float32, seed=sum(shape) + 5)
+    dy = torch.randn(shape, generator=torch.Generator().manual_seed(12))
+    y_ref, g_ref = _oracle(pre, dy, compute)
+    y, grads = _run(pre, dy, gpu, torch.float32, compute_dtype=compute)
+    assert y.dtype == torch.float32
+    # 16-bit compute: a gate within an fp32 ulp of a rounding tie rounds the other way than the float64 oracle's, so y
+    # carries differences the size of the compute dtype's spacing; fp32 compute meets the fp32 bar but for the
+    # hardware's 1-ulp exp and reciprocal inside the sigmoids
+    tol = {torch.float32: 2e-5, torch.float16: 1e-3, torch.bfloat16: 1e-2}[compute]
+    assert_close("y", y, y_ref, tol)
+    for name, got, want in zip(NAMES, grads, g_ref):
+        assert got.dtype == torch.float32
+        assert_close(name, got, want, 2e-5 if compute == torch.float32 else 1e-2)
+
+
+def test_gated_scan_over_fp32_projections_equals_prologue_plus_scan(gpu):
+    # the same values through the two-pass route (gate prologue kernel, then the plain scan on fp16 operands with
+    # fp32 y): the operands are the same bits, so y differs by the order of the fp32 sums only (another tile
+    # geometry); gradients to the rounding of the activations' derivatives
+    shape, compute = (2, 900, 384), torch.float16
+    pre = _projections(shape, torch.float32, seed=4)
+    dy = torch.randn(shape, generator=torch.Generator().manual_seed(13))
+    y, grads = _run(pre, dy, gpu, torch.float32, compute_dtype=compute)
+    leaves = [t.to(gpu).requires_grad_(True) for t in pre]
+    a, x, c, b = gate_prologue(*leaves, compute)
+    y2 = scan(x, a, b, c, out_dtype=torch.float32)
+    y2.backward(dy.to(gpu))
+    assert_close("y", y, y2.detach().cpu().double().numpy(), 1e-5)
+    for name, got, leaf in zip(NAMES, grads, leaves):
+        assert_close(name, got, leaf.grad.cpu().double().numpy(), 1e-2)
+
+
+def test_gated_scan_over_fp32_projections_as_blocks_of_one_wide_tensor(gpu):
+    # the five fp32 projections as column blocks of one [B, L, 5 S] GEMM output, gradients into one wide tensor:
+    # the same launches on strided views, so the same bits as the five-tensor entry
+    B, L, S, compute = 2, 500, 256, torch.bfloat16
+    pre = _projections((B, L, S), torch.float32, seed=18)
+    dy = torch.randn((B, L, S), generator=torch.Generator().manual_seed(14)).to(gpu)
+    leaves = [t.to(gpu).requires_grad_(True) for t in pre]
+    y = gated_scan.gated_scan(*leaves, out_dtype=torch.float32, compute_dtype=compute)
+    y.backward(dy)
+    wide = torch.cat(pre, dim=-1).to(gpu).requires_grad_(True)
+    assert gated_scan.supported([wide[..., k * S:(k + 1) * S] for k in range(5)], compute, torch.float32)
+    y_w = gated_scan.gated_scan_wide(wide, out_dtype=torch.float32, compute_dtype=compute)
+    y_w.backward(dy)
+    assert hip_scan.workspace_status() == 0
+    assert torch.equal(y, y_w)
+    for k, leaf in enumerate(leaves):
+        assert torch.equal(wide.grad[..., k * S:(k + 1) * S], leaf.grad), NAMES[k]
 
 
 def test_gated_scan_with_fp32_y_takes_the_two_pass_backward(gpu):
@@ -123,7 +182,11 @@ def test_what_the_gated_launches_do_not_take(gpu):
     assert gated_scan.supported(pre, torch.bfloat16, torch.bfloat16)
     assert not gated_scan.supported(pre, torch.float16, torch.float16)              # compute dtype differs from storage
     assert not gated_scan.supported(pre, torch.bfloat16, torch.bfloat16, checkpoint=False)
-    assert not gated_scan.supported([t.float() for t in pre], torch.float32, torch.float32)
+    wide32 = [t.float() for t in pre]
+    assert gated_scan.supported(wide32, torch.float32, torch.float32)               # fp32 projections: any compute dtype,
+    assert gated_scan.supported(wide32, torch.float16, torch.float32)               # fp32 y only
+    assert not gated_scan.supported(wide32, torch.float16, torch.float16)
+    assert not gated_scan.supported([t[..., 2:] for t in wide32], torch.float16, torch.float32)   # rows off 16 bytes
     assert not gated_scan.supported([t[..., :100] for t in pre], torch.bfloat16, torch.bfloat16)     # S < 128
     assert not gated_scan.supported([t[..., 4:] for t in pre], torch.bfloat16, torch.bfloat16)       # rows off 16 bytes
     assert not gated_scan.supported([t.cpu() for t in pre], torch.bfloat16, torch.bfloat16)
