@@ -460,6 +460,17 @@ QSSM_API int qssm_rmsnorm_backward(const void* dy, int64_t ld_dy, const void* x,
                           int64_t rows, int32_t H, float eps, int32_t dtype, void* stream);
 
 /*
+ * Column sums of a [rows, S] matrix with row stride `ld` (elements; a column block of a wider matrix is fine):
+ * out[s] = sum over r of x[r, s], accumulated in fp32 in a fixed order (results repeat bit for bit) and stored in
+ * x's storage type.  `partial` is fp32 scratch of `partial_rows` x S floats (64 rows suit a few thousand rows of x;
+ * more rows of x per row of scratch only make the first of the two launches longer).
+ * This is the bias gradient of a linear map, which autograd otherwise computes with a library reduction per bias:
+ * replaces what autograd records for the `+ bias` of A_proj and out_proj, quick_ssm/layers.py:50-58,76,106.
+ */
+QSSM_API int qssm_colsum(const void* x, int64_t ld, int64_t rows, int32_t S, int32_t dtype, float* partial,
+                         int32_t partial_rows, void* out, void* stream);
+
+/*
  * Streaming copy of `bytes` bytes (16-byte aligned, multiple of 16) on `stream`.  Not part of
  * the scan: it is the known-size kernel against which rocprof's FETCH_SIZE / WRITE_SIZE
  * counters and the achievable-bandwidth ceiling are calibrated by the benchmark.

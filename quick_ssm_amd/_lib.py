@@ -45,6 +45,7 @@ EXPORTED_SYMBOLS = (
     "qssm_gates_backward_strided",
     "qssm_rmsnorm_forward",
     "qssm_rmsnorm_backward",
+    "qssm_colsum",
     "qssm_copy_bytes",
     "qssm_launch_count_step",
 )
@@ -187,6 +188,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.qssm_rmsnorm_forward.argtypes = [vp, i64, vp, vp, vp, i64, i32, ctypes.c_float, i32, vp]
     lib.qssm_rmsnorm_backward.restype = ctypes.c_int
     lib.qssm_rmsnorm_backward.argtypes = [vp, i64, vp, i64, vp, vp, vp, vp, vp, i32, i64, i32, ctypes.c_float, i32, vp]
+    lib.qssm_colsum.restype = ctypes.c_int
+    lib.qssm_colsum.argtypes = [vp, i64, i64, i32, i32, vp, i32, vp, vp]
     lib.qssm_copy_bytes.restype = ctypes.c_int
     lib.qssm_copy_bytes.argtypes = [vp, vp, u64, vp]
     lib.qssm_launch_count_step.restype = ctypes.c_int

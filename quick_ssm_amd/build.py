@@ -18,7 +18,7 @@ PKG_DIR = Path(__file__).resolve().parent
 SRC_DIR = PKG_DIR / "csrc"
 OBJ_DIR = SRC_DIR / "build"
 LIB_PATH = PKG_DIR / "libquick_ssm_hip.so"
-SOURCES = ("scan_fwd.hip", "scan_bwd.hip", "gates.hip", "rmsnorm.hip", "scan_api.hip")
+SOURCES = ("scan_fwd.hip", "scan_bwd.hip", "gates.hip", "rmsnorm.hip", "colsum.hip", "scan_api.hip")
 
 # Packed-fp32 VALU forms are kept out of the generated code on purpose.
 HIPCC_FLAGS = [

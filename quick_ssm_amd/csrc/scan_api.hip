@@ -899,6 +899,26 @@ extern "C" int qssm_scan_forward_static(const qssm_plan* plan, const void* x, qs
 
 extern "C" {
 
+int qssm_colsum(const void* x, int64_t ld, int64_t rows, int32_t S, int32_t dtype, float* partial, int32_t partial_rows,
+                void* out, void* stream) {
+  const int es = dtype_size(dtype);
+  if (es == 0) return fail(QSSM_EINVAL, "unknown dtype code");
+  if (rows < 0 || S < 0) return fail(QSSM_EINVAL, "negative dimension");
+  if (S == 0) return 0;
+  if (!out || !partial || (rows > 0 && !x)) return fail(QSSM_EINVAL, "NULL tensor");
+  if (ld < S) return fail(QSSM_EINVAL, "row stride below S");
+  if (partial_rows < 1) return fail(QSSM_EINVAL, "partial needs at least one row of S floats");
+  // about 64 rows per chunk, as many chunks as `partial` has rows for
+  int64_t chunks = (rows + 63) / 64;
+  if (chunks > partial_rows) chunks = partial_rows;
+  if (chunks < 1) chunks = 1;
+  const int vec = rows == 0 ? 1 : gate_vec(S, {{x, ld}}, es, {}, es);
+  if (!launch_colsum_any(dtype, x, ld, rows, S, vec, partial, (int)chunks, out, (hipStream_t)stream))
+    return fail(QSSM_EINVAL, "column sum for storage type %d is not built", dtype);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : hip_fail(e, "colsum kernel launch");
+}
+
 int qssm_launch_count_step(uint32_t count, int32_t static_scratch, uint32_t* flag, uint32_t* next, int32_t* wipes) {
   if (flag == nullptr || next == nullptr || wipes == nullptr) return fail(QSSM_EINVAL, "NULL argument");
   const unsigned reset_at = static_scratch ? kScratchWipeAt : kCountWrapAt;

@@ -554,4 +554,9 @@ struct NormBwdArgs {
 bool launch_norm_any(int dtype, const NormFwdArgs* f, const NormBwdArgs* b, int vec, int max_partial_rows, void* dw,
                      hipStream_t stream);
 
+// ---- column sums (colsum.hip): bias gradients of the layer's linear maps ---------------------------------------
+// `partial` holds `chunks` rows of S floats.  False if the storage type is not built.
+bool launch_colsum_any(int dtype, const void* x, int64_t ld, int64_t rows, int S, int vec, float* partial, int chunks,
+                       void* out, hipStream_t stream);
+
 }  // namespace qssm

@@ -16,6 +16,7 @@ from typing import Optional
 import torch
 import torch.nn as nn
 
+from . import _lib
 from . import gated_scan as _gated
 from . import scan_interface as _scan_interface
 from .gates import gate_prologue, gate_prologue_wide
@@ -33,6 +34,46 @@ class RMSNorm(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return rms_norm(x, self.weight, self.eps)
+
+
+_CODES = {torch.float32: _lib.QSSM_F32, torch.float16: _lib.QSSM_F16, torch.bfloat16: _lib.QSSM_BF16}
+_COLSUM_PARTIAL_ROWS = 64
+
+
+def column_sum(g2: torch.Tensor) -> torch.Tensor:
+    """Sum over the rows of a [rows, S] matrix: the bias gradient of a linear map from its output's gradient.
+
+    GPU matrices with unit column stride (a column block of a wider matrix is fine) take `qssm_colsum`: two small
+    launches, a fixed summation order; a library reduction of this shape costs as much as the layer's scan at the
+    copy task's size.  Everything else is `g2.sum(0)`."""
+    rows, S = g2.shape
+    if not (g2.is_cuda and g2.dtype in _CODES and S > 0 and rows > 0 and g2.stride(1) == 1 and g2.stride(0) >= S):
+        return g2.sum(0)
+    out = torch.empty((S,), dtype=g2.dtype, device=g2.device)
+    partial = torch.empty((_COLSUM_PARTIAL_ROWS, S), dtype=torch.float32, device=g2.device)
+    with _lib.launch_stream(g2.device) as stream:
+        _lib.check(_lib.load().qssm_colsum(g2.data_ptr(), g2.stride(0), rows, S, _CODES[g2.dtype], partial.data_ptr(),
+                                           _COLSUM_PARTIAL_ROWS, out.data_ptr(), stream))
+    return out
+
+
+class _LinearBias(torch.autograd.Function):
+    """u @ weight^T + bias, as `torch.nn.functional.linear`, with the bias gradient from `column_sum`."""
+
+    @staticmethod
+    def forward(ctx, u, weight, bias):
+        ctx.save_for_backward(u, weight)
+        return torch.nn.functional.linear(u, weight, bias)
+
+    @staticmethod
+    def backward(ctx, g):
+        u, weight = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        g2 = g.reshape(-1, g.shape[-1])
+        du = (g2 @ weight).view_as(u) if need[0] else None
+        dw = g2.t() @ u.reshape(-1, u.shape[-1]) if need[1] else None
+        db = column_sum(g2) if need[2] else None
+        return du, dw, db
 
 
 class _PackedProjection(torch.autograd.Function):
@@ -57,7 +98,7 @@ class _PackedProjection(torch.autograd.Function):
         if any(need[1:6]):
             dw = g2.t() @ u.reshape(-1, u.shape[-1])                              # [5 S, H]
             blocks = [dw[k * S:(k + 1) * S] if need[1 + k] else None for k in range(5)]
-        dbias = g2[:, :S].sum(0) if need[6] else None
+        dbias = column_sum(g2[:, :S]) if need[6] else None
         return (du, *blocks, dbias, None, None)
 
 
@@ -190,7 +231,8 @@ class SSM(nn.Module):
                     forget, drive, out_gate, in_gate = gate_prologue(*pre, self.compute_dtype)
                 y = scan(x=drive, a=forget, b=in_gate, c=out_gate, block_l=block_l, checkpoint=checkpoint,
                          tile_b=tile_b, tile_d=tile_d, out_dtype=out_dtype, backend=backend)
-            return self.out_proj(y.to(w_dtype)) + skip
+            y = y if y.dtype == w_dtype else y.to(w_dtype)
+            return _LinearBias.apply(y, self.out_proj.weight, self.out_proj.bias) + skip
         drive, forget, in_gate, out_gate = self.gates(u)
         y = scan(
             x=drive, a=forget, b=in_gate, c=out_gate,
