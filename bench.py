@@ -176,10 +176,35 @@ def record_traffic(fetch_csv: str, write_csv: str, workload: str) -> int:
     write = mean_kib(write_csv, "WRITE_SIZE", "scan_bwd") * copy_kib / mean_kib(write_csv, "WRITE_SIZE", "copy_kernel")
     rec = {"kernel": "scan_bwd_kernel", "workload": workload, "traffic_bytes_per_launch": int(fetch * 1024) + int(write * 1024),
            "fetch_bytes": int(fetch * 1024), "write_bytes": int(write * 1024), "kernel_source_hash": kernel_source_hash(),
-           "source": f"profiles/scan_{workload}_bf16_hbm_traffic.md" if workload == "c1" else "rocprofv3 FETCH_SIZE / WRITE_SIZE"}
+           "source": f"profiles/scan_{workload}_{ {'float32': 'f32', 'float16': 'fp16', 'bfloat16': 'bf16'}[dt_name] }_hbm_traffic.md"}
     out = ROOT / "profiles" / f"scan_bwd_{workload}_traffic.json"
     out.write_text(json.dumps(rec, indent=1))
     print(json.dumps(rec))
+    return 0
+
+
+def settle_timeline(torch, step) -> int:
+    """Per-step durations (HIP events between the steps) of 60 steps begun right after idle spells of different
+    lengths, printed as text: how long the device takes to settle after a pause, and from which pause on."""
+    def timeline(n):
+        torch.cuda.synchronize()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(n + 1)]
+        ev[0].record()
+        for k in range(n):
+            step()
+            ev[k + 1].record()
+        torch.cuda.synchronize()
+        return [ev[k].elapsed_time(ev[k + 1]) * 1e3 for k in range(n)]
+
+    for _ in range(100):     # 30 ms and more of load first: the settled rate
+        step()
+    base = timeline(60)
+    print(f"settled: mean of 60 steps {sum(base[1:]) / 59:.1f} us (first step after the synchronize: {base[0]:.0f} us)")
+    for idle_ms in (2, 5, 10, 20, 50, 200):
+        time.sleep(idle_ms * 1e-3)
+        per = timeline(60)
+        print(f"after {idle_ms:3d} ms idle: steps 2-10 {sum(per[1:10]) / 9:.1f} us, 11-20 {sum(per[10:20]) / 10:.1f}, "
+              f"21-30 {sum(per[20:30]) / 10:.1f}, 31-60 {sum(per[30:]) / 30:.1f} | " + " ".join(f"{p:.0f}" for p in per[:40]), flush=True)
     return 0
 
 
@@ -192,6 +217,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--settle-timeline", action="store_true",
+                    help="instead of the benchmark: per-step times of the steps that follow idle spells of 2 to 200 ms "
+                         "(what the untimed run-in in front of the measurements is for)")
     args = ap.parse_args()
     if args.record_traffic:
         return record_traffic(args.record_traffic[0], args.record_traffic[1], args.workload)
@@ -248,6 +276,9 @@ def main() -> int:
         # hand-over costs more than the launch it brackets when the workload is small; it changes nothing on the GPU)
         with torch.autograd.set_multithreading_enabled(False):
             y.backward(gy)
+
+    if args.settle_timeline:
+        return settle_timeline(torch, step)
 
     # ---- everything the run needs exists before the first measured launch ------------------------
     # An allocation of this size is milliseconds of idle GPU, and an idle spell of 10 ms or more is followed by
