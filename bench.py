@@ -269,13 +269,15 @@ def main() -> int:
     def step():
         ops, gy = sets[turn[0] % n_sets]
         turn[0] += 1
-        for t in ops:
-            t.grad = None
         y = scan(*ops, block_l=block_l, checkpoint=True, out_dtype=out_dtype)
         # one device, one graph: run the backward on this thread instead of waking autograd's device thread (the
         # hand-over costs more than the launch it brackets when the workload is small; it changes nothing on the GPU)
         with torch.autograd.set_multithreading_enabled(False):
             y.backward(gy)
+        # gradients are dropped at the end of the step, as a training loop's zero_grad(set_to_none=True) does: the
+        # next step starts with its forward launch
+        for t in ops:
+            t.grad = None
 
     if args.settle_timeline:
         return settle_timeline(torch, step)
@@ -340,16 +342,21 @@ def main() -> int:
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = wall_ms
+    # the same K steps once more between two HIP events, for the GPU's own clock beside the host's (the headline is
+    # the wall clock above; events inside that region would only add host work in front of its first launch)
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     ev0.record()
     for _ in range(args.steps):
         step()
     ev1.record()
     torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     gpu_ms = ev0.elapsed_time(ev1) / args.steps
-    ms_per_step = wall_ms
 
     # the same K steps right after an idle spell, no warm-up: what a job that leaves the device idle between steps sees
     time.sleep(IDLE_MS * 1e-3)

@@ -343,13 +343,14 @@ _plans: Dict[tuple, Plan] = {}
 _forward_keep = True
 
 
-def set_forward_keep(flag: bool) -> bool:
+def set_forward_keep(flag):
     """Whether forwards planned from now on follow the planner's cache policy (`plan.keep_tiles`: the last tiles of
-    every chain load their operands with ordinary loads, for a backward that starts there) or stream every operand
-    past the caches (False).  Results are the same bit for bit; only what a launch leaves in the caches differs.
-    Returns the old setting."""
+    every chain load their operands with ordinary loads, for a backward that starts there; True), stream every
+    operand past the caches (False), or keep at most that many tiles per chain (an int).  Results are the same bit
+    for bit; only what a launch leaves in the caches differs.  Returns the old setting."""
     global _forward_keep
-    old, _forward_keep = _forward_keep, bool(flag)
+    old = _forward_keep
+    _forward_keep = flag if isinstance(flag, bool) else max(0, int(flag))
     return old
 
 
@@ -472,9 +473,9 @@ def scan_forward(
             # The backward decides how far apart the saved states may be; the forward follows.
             stride = make_plan(B, L, D, in_dtype, out_dtype, _lib.QSSM_BACKWARD, align, 0, bwd_tune).seg_len
         plan = make_plan(B, L, D, in_dtype, out_dtype, _lib.QSSM_FORWARD, align, stride, tune)
-        if not keep:
+        if keep is not True:
             plan = Plan.from_buffer_copy(plan)   # cached plans are shared: change a copy
-            plan.keep_tiles = 0
+            plan.keep_tiles = 0 if keep is False else min(int(plan.keep_tiles), int(keep))
         return _Launch(plan, ForwardCall())
 
     entry = _launch_entry((0, B, L, D, in_dtype, out_dtype, align, want_ckpt, tune, bwd_tune, keep), make)
