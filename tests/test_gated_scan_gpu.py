@@ -127,6 +127,39 @@ def test_gated_scan_over_fp32_projections_as_blocks_of_one_wide_tensor(gpu):
         assert torch.equal(wide.grad[..., k * S:(k + 1) * S], leaf.grad), NAMES[k]
 
 
+@pytest.mark.timeout(600)
+def test_gated_scan_over_a_wide_tensor_past_4_gib(gpu):
+    # [32, 2048, 5 x 4096] fp32 is 5 GiB: the projections of the last batch rows lie past 2^32 bytes.  Drawn on the
+    # device; windows of columns of the first and the last batch row go to the float64 oracle composition.
+    B, L, S, compute = 32, 2048, 4096, torch.float16
+    free, _ = torch.cuda.mem_get_info(gpu)
+    if free < (40 << 30):
+        pytest.skip("needs 40 GiB of free device memory")
+    print("case gated scan over 5 GiB of projections", flush=True)
+    gen = torch.Generator(device=gpu).manual_seed(23)
+    wide = torch.empty((B, L, 5 * S), dtype=torch.float32, device=gpu).normal_(generator=gen)
+    wide[..., 0 * S:1 * S].mul_(0.8).add_(3.0)
+    wide[..., 2 * S:3 * S].mul_(1.5)
+    wide[..., 4 * S:5 * S].mul_(1.5).sub_(1.0)
+    wide.requires_grad_(True)
+    dy = torch.empty((B, L, S), dtype=torch.float32, device=gpu).normal_(generator=gen)
+    assert gated_scan.supported([wide[..., k * S:(k + 1) * S] for k in range(5)], compute, torch.float32)
+    y = gated_scan.gated_scan_wide(wide, out_dtype=torch.float32, compute_dtype=compute)
+    y.backward(dy)
+    assert hip_scan.workspace_status() == 0
+    assert bool(torch.isfinite(y).all()) and bool(torch.isfinite(wide.grad).all())
+    for row in (0, B - 1):
+        for c0 in (0, S - 64):
+            pre = [wide.detach()[row:row + 1, :, k * S + c0:k * S + c0 + 64].cpu() for k in range(5)]
+            y_ref, g_ref = _oracle(pre, dy[row:row + 1, :, c0:c0 + 64].cpu(), compute)
+            assert_close(f"y[row {row}, cols {c0}]", y[row:row + 1, :, c0:c0 + 64].detach().cpu(), y_ref, 1e-2)
+            for k, (name, ref) in enumerate(zip(NAMES, g_ref)):
+                got = wide.grad[row:row + 1, :, k * S + c0:k * S + c0 + 64].cpu()
+                assert_close(f"{name}[row {row}, cols {c0}]", got, ref, 1e-2)
+    del y, dy, wide
+    torch.cuda.empty_cache()
+
+
 def test_gated_scan_with_fp32_y_takes_the_two_pass_backward(gpu):
     # y stored as fp32 (the layer's scan_out_dtype): forward fused, backward through the prologue and the plain scan
     shape, dtype = (2, 600, 256), torch.float16

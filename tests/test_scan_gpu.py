@@ -707,6 +707,43 @@ def test_config1_bf16_full_shape(gpu):
 
 
 @pytest.mark.timeout(600)
+def test_tensors_past_4_gib_reach_their_last_batch_row(gpu):
+    # 5 x 8192 x 65536 bf16 is 5 GiB per tensor: the last batch row starts 2^31 elements = 2^32 bytes into each of
+    # them, past what 32-bit offsets reach.  Operands are drawn on the device; windows of columns of the first, the
+    # fourth and the last row go to the float64 oracle.
+    B, L, D = 5, 8192, 65536
+    free, _ = torch.cuda.mem_get_info(gpu)
+    if free < (80 << 30):
+        pytest.skip("needs 80 GiB of free device memory")
+    print("case tensors of 5 GiB", flush=True)
+    gen = torch.Generator(device=gpu).manual_seed(7)
+
+    def new():
+        return torch.empty((B, L, D), dtype=torch.bfloat16, device=gpu)
+
+    x = new().normal_(generator=gen)
+    a = new().uniform_(0.9, 1.0, generator=gen)
+    b = new().normal_(0.0, 0.1, generator=gen)
+    c = new().uniform_(0.0, 1.0, generator=gen)
+    dy = new().normal_(generator=gen)
+    leaves = [t.requires_grad_(True) for t in (x, a, b, c)]
+    y = scan(*leaves, block_l=256, checkpoint=True)
+    y.backward(dy)
+    assert hip_scan.workspace_status() == 0
+    got = {"y": y.detach(), "dx": x.grad, "da": a.grad, "db": b.grad, "dc": c.grad}
+    for k, t in got.items():
+        assert t.shape == (B, L, D) and bool(torch.isfinite(t).all()), k
+    for row in (0, 3, B - 1):
+        for c0 in (0, D // 2 - 32, D - 64):
+            win = (slice(row, row + 1), slice(None), slice(c0, c0 + 64))
+            ref = oracle_all(*(t.detach()[win].cpu() for t in (x, a, b, c, dy)))
+            for k in ("y", "dx", "da", "db", "dc"):
+                assert_close(f"{k}[row {row}, cols {c0}:{c0 + 64}]", got[k][win].cpu(), ref[k], TOL[torch.bfloat16])
+    del got, y, leaves, x, a, b, c, dy
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.timeout(600)
 def test_config2_fp16_long_sequence_near_unit_decay(gpu):
     # B=1 L=65536 D=4096 fp16, a in [0.99, 1], block_l=1024, tile_d=1024: every column over all of L, the oracle
     # taking 512 columns at a time
