@@ -661,6 +661,28 @@ def test_partial_gradients(gpu):
     assert_close("dc", cs.grad, ref["dc"], 1e-5)
 
 
+def test_float64_operands_run_in_fp32_and_come_back_as_float64(gpu):
+    # quick_ssm/triton_forwards.py:7-16 casts whatever float type it gets to fp32; y comes back in x.dtype
+    # (scan_interface.py:200) and every gradient in its operand's dtype (:148-151)
+    x, a, b, c, dy = (t.double() for t in make_inputs((2, 300, 24), seed=21))
+    ref = oracle_all(x, a, b, c, dy)
+    got = run_scan_with_grads(scan, x, a, b, c, dy, gpu)
+    for k in ("y", "dx", "da", "db", "dc"):
+        assert got[k].dtype == torch.float64, k
+        assert_close(k, got[k], ref[k], 1e-5)
+    # mixed storage: the operands meet in the widest type among them, each gradient returns in its own
+    leaves = [t.to(gpu).requires_grad_(True) for t in (x.half(), a.float(), b.bfloat16(), c.double())]
+    y = scan(*leaves, out_dtype=torch.float32)
+    y.backward(dy.to(gpu).float())
+    assert y.dtype == torch.float32
+    for t in leaves:
+        assert t.grad.dtype == t.dtype and bool(torch.isfinite(t.grad).all())
+    ref = oracle_all(x.half().double(), a.float().double(), b.bfloat16().double(), c, dy.float().double())
+    assert_close("y", y, ref["y"], 1e-5)
+    assert_close("da", leaves[1].grad, ref["da"], 1e-5)
+    assert_close("dx", leaves[0].grad, ref["dx"], 1e-2)
+
+
 def test_argument_errors(gpu):
     x = torch.zeros(2, 8, 4, device=gpu)
     with pytest.raises(ValueError):
