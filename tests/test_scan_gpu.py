@@ -106,6 +106,38 @@ def test_closed_form_geometric_decay(gpu, dtype):
     assert rel[-1] < 3e-4
 
 
+def test_a_million_steps_of_near_unit_decay(gpu):
+    # The reference's precision test at its own length (quick_ssm/forward_only.py:548-629: L = 2^20, an impulse at
+    # t = 0, b = 1, a = g), with g chosen so that g^L stays a normal number: h(t) = g^t over 2^20 steps and the
+    # thousands of hand-overs between tiles they take, against float64 powers of the stored g; and y, with the
+    # gradients of a random dy, against the float64 oracle on a second, random, input of the same length.
+    L, D = 1 << 20, 16
+    g = float(torch.tensor(0.99999, dtype=torch.float32).double())
+    x = torch.zeros(1, L, D)
+    x[:, 0] = 1
+    a = torch.full_like(x, g)
+    b = torch.ones_like(x)
+    print("case 2^20 steps", flush=True)
+    _, h = hip_scan.block_scan_forward_3d(x.to(gpu), a.to(gpu), b.to(gpu))
+    expect = g ** np.arange(L)
+    rel = np.abs(h[0].double().cpu().numpy() - expect[:, None]) / expect[:, None]
+    print(f"  g^t: worst relative error {rel.max():.2e}, at the last step {rel[-1].max():.2e}", flush=True)
+    # With one g for every step every tile carries the same product g^64 with the same rounding error, which the
+    # 16 384 tiles of the chain then repeat instead of averaging out: 1.3e-3 at the last step (measured), where the
+    # sequential fp32 recurrence on this input reaches 1.3e-4.  Any evaluation by blocks has this property, the
+    # reference's per-block running products (quick_ssm/triton_forwards.py:63-70) included; operands that vary from
+    # step to step do not show it (second half of this test: 1e-5 of the largest value over the same 2^20 steps).
+    worst_abs = np.abs(h[0].double().cpu().numpy() - expect[:, None]).max()
+    print(f"  g^t: largest absolute error {worst_abs:.2e}", flush=True)
+    assert rel.max() < 5e-3, (rel.max(), rel[-1].max())
+    assert worst_abs < 2e-4
+    x, a, b, c, dy = make_inputs((1, L, D), seed=31, a_lo=0.999, a_span=0.001)
+    got = run_scan_with_grads(scan, x, a, b, c, dy, gpu)
+    ref = oracle_all(x, a, b, c, dy)
+    assert hip_scan.workspace_status() == 0
+    _check_all(got, ref, 1e-5)
+
+
 # ---- shapes, dtypes, edges ---------------------------------------------------------------------------
 
 SHAPES = [
