@@ -84,14 +84,19 @@ def _launch(plan: Plan, dev: torch.device, fn, *args) -> None:
         hip_scan._after_launch(buf, stream, capturing)
 
 
-def _forward_launch(pre: Sequence[Tensor], compute_dtype: torch.dtype, out_dtype: torch.dtype):
-    """y, the saved states and their spacing for the five projection outputs."""
+def _forward_launch(pre: Sequence[Tensor], compute_dtype: torch.dtype, out_dtype: torch.dtype, train: bool = True):
+    """y, the saved states and their spacing for the five projection outputs.  `train`: a backward will follow, so
+    the last tiles of every chain may leave their operands in the caches for it (`hip_scan.set_forward_keep`)."""
     A_pre, B_in, Ca, Cb, D_pre = pre
     B, L, S = A_pre.shape
     dev, dtype = A_pre.device, A_pre.dtype
     # the backward's tile length decides how far apart the saved states are; it takes dy stored as the projections are
     stride = _plan(B, L, S, dtype, compute_dtype, dtype, _lib.QSSM_BACKWARD, 0).seg_len
     plan = _plan(B, L, S, dtype, compute_dtype, out_dtype, _lib.QSSM_FORWARD, stride)
+    keep = hip_scan._forward_keep if train else False
+    if keep is not True:
+        plan = Plan.from_buffer_copy(plan)   # cached plans are shared: change a copy
+        plan.keep_tiles = 0 if keep is False else min(int(plan.keep_tiles), int(keep))
     y = torch.empty((B, L, S), dtype=out_dtype, device=dev)
     ckpt = torch.empty((B, plan.n_ckpt, S), dtype=torch.float32, device=dev)
     _launch(plan, dev, _lib.load().qssm_scan_gated_forward,
@@ -127,7 +132,8 @@ class _GatedScanFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, A_pre: Tensor, B_in: Tensor, Ca: Tensor, Cb: Tensor, D_pre: Tensor, out_dtype: torch.dtype,
                 compute_dtype: torch.dtype) -> Tensor:
-        y, ckpt, stride = _forward_launch((A_pre, B_in, Ca, Cb, D_pre), compute_dtype, out_dtype)
+        y, ckpt, stride = _forward_launch((A_pre, B_in, Ca, Cb, D_pre), compute_dtype, out_dtype,
+                                          any(ctx.needs_input_grad[:5]))
         ctx.save_for_backward(A_pre, B_in, Ca, Cb, D_pre, ckpt)
         ctx.stride, ctx.out_dtype, ctx.compute_dtype = stride, out_dtype, compute_dtype
         return y
@@ -158,7 +164,7 @@ class _GatedScanWide(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, wide: Tensor, out_dtype: torch.dtype, compute_dtype: torch.dtype) -> Tensor:
-        y, ckpt, stride = _forward_launch(_blocks(wide), compute_dtype, out_dtype)
+        y, ckpt, stride = _forward_launch(_blocks(wide), compute_dtype, out_dtype, ctx.needs_input_grad[0])
         ctx.save_for_backward(wide, ckpt)
         ctx.stride, ctx.out_dtype, ctx.compute_dtype = stride, out_dtype, compute_dtype
         return y

@@ -465,7 +465,8 @@ def scan_forward(
 
     (x, a, b, c), strides, ptrs, align = _describe((x, a, b, c), (y, h), L, D)
 
-    keep = _forward_keep
+    # Operands are left in the caches only for a backward: a forward that saves no states has none coming.
+    keep = _forward_keep if (want_ckpt or want_h) else False
 
     def make() -> _Launch:
         stride = 0

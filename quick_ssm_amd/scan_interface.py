@@ -99,14 +99,17 @@ class _HipScanFunction(torch.autograd.Function):
         ctx.tile_states = []
         whole = len(tiles) == 1
         y = None if whole else torch.empty(x.shape, dtype=k_out, device=x.device)
+        # No operand wants a gradient (inference, torch.no_grad()): no backward will come, so no state is saved and
+        # the launch streams its operands past the caches.
+        train = any(ctx.needs_input_grad[:4])
         h_saved = None
-        if not checkpoint and not whole:
+        if train and not checkpoint and not whole:
             h_saved = torch.empty(x.shape, dtype=torch.float32, device=x.device)
         for bs_, ds_ in tiles:
             # the common case, one launch over the whole tensor, skips four view constructions
             ops = (xs, as_, bs, cs) if whole else tuple(t[bs_, :, ds_] for t in (xs, as_, bs, cs))
             yt, ht, ckpt, stride = hip_scan.scan_forward(
-                *ops, out_dtype=k_out, want_h=not checkpoint, want_ckpt=bool(checkpoint),
+                *ops, out_dtype=k_out, want_h=train and not checkpoint, want_ckpt=train and bool(checkpoint),
             )
             ctx.tile_states.append((ckpt, stride))
             if whole:
@@ -193,8 +196,9 @@ class _HipScanCarryFunction(torch.autograd.Function):
             if h0.data_ptr() % 16 != 0:
                 h0 = h0.clone()
         h_final = torch.empty((B, D), dtype=torch.float32, device=x.device)
+        train = any(ctx.needs_input_grad[:5])   # generation mode saves no states and leaves nothing in the caches
         y, h_full, ckpt, stride = hip_scan.scan_forward(
-            xs, as_, bs, cs, out_dtype=k_out, want_h=not checkpoint, want_ckpt=bool(checkpoint),
+            xs, as_, bs, cs, out_dtype=k_out, want_h=train and not checkpoint, want_ckpt=train and bool(checkpoint),
             h_init=h0, h_final=h_final,
         )
         ctx.save_for_backward(x, a, b, c)

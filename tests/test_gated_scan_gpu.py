@@ -160,6 +160,17 @@ def test_gated_scan_over_a_wide_tensor_past_4_gib(gpu):
     torch.cuda.empty_cache()
 
 
+def test_gated_forward_without_a_backward_equals_the_one_with(gpu):
+    # no projection wants a gradient: the launch is planned with keep_tiles = 0; y is the same bit for bit
+    pre = [t.to(gpu) for t in _projections((2, 900, 512), torch.bfloat16, seed=41)]
+    with torch.no_grad():
+        y0 = gated_scan.gated_scan(*pre, out_dtype=torch.bfloat16)
+    y1 = gated_scan.gated_scan(*[t.clone().requires_grad_(True) for t in pre], out_dtype=torch.bfloat16)
+    assert y0.grad_fn is None and y1.grad_fn is not None
+    assert torch.equal(y0, y1.detach())
+    assert hip_scan.workspace_status() == 0
+
+
 def test_gated_scan_with_fp32_y_takes_the_two_pass_backward(gpu):
     # y stored as fp32 (the layer's scan_out_dtype): forward fused, backward through the prologue and the plain scan
     shape, dtype = (2, 600, 256), torch.float16

@@ -682,6 +682,35 @@ def test_launch_geometry_does_not_change_results_beyond_rounding(gpu):
     assert hip_scan.workspace_status() == 0
 
 
+def test_a_forward_that_no_backward_follows_saves_no_states(gpu, monkeypatch):
+    # inference (no operand wants a gradient, or torch.no_grad()): same y bit for bit, no saved states, and the launch
+    # is planned to stream its operands past the caches (plan.keep_tiles = 0)
+    seen = []
+    real = hip_scan.scan_forward
+
+    def spy(*args, **kw):
+        out = real(*args, **kw)
+        seen.append((kw.get("want_h"), kw.get("want_ckpt"), out[2]))
+        return out
+
+    monkeypatch.setattr(hip_scan, "scan_forward", spy)
+    x, a, b, c, _ = make_inputs((2, 700, 256), dtype=torch.bfloat16, seed=3)
+    ops = [t.to(gpu) for t in (x, a, b, c)]
+    with torch.no_grad():
+        y0 = scan(*ops)
+    assert seen[-1][:2] == (False, False) and seen[-1][2] is None and y0.grad_fn is None
+    y1 = scan(*ops)                                   # grad mode on, but no operand requires a gradient
+    assert seen[-1][:2] == (False, False) and seen[-1][2] is None
+    leaves = [t.clone().requires_grad_(True) for t in ops]
+    y2 = scan(*leaves)
+    assert seen[-1][:2] == (False, True) and seen[-1][2] is not None
+    assert torch.equal(y0, y1) and torch.equal(y0, y2.detach())
+    with torch.no_grad():
+        y3, state = scan_chunk(*ops, state=None)
+    assert seen[-1][:2] == (False, False) and torch.equal(y3, y0)
+    assert hip_scan.workspace_status() == 0
+
+
 def test_partial_gradients(gpu):
     x, a, b, c, dy = make_inputs((2, 400, 16), seed=9)
     ref = oracle_all(x, a, b, c, dy)
