@@ -7,4 +7,4 @@ from .scan_interface import scan, scan_chunk
 from .layers import SSM, RMSNorm
 
 __all__ = ["scan", "scan_chunk", "SSM", "RMSNorm"]
-__version__ = "0.1.0"
+__version__ = "0.2.0"
