@@ -229,11 +229,18 @@ int qssm_plan_scan_gated(int32_t B, int32_t L, int32_t D, int32_t dtype, int32_t
   if (D % 4 != 0 || (align_elems * es) % 16 != 0 || D < 128)
     return fail(QSSM_EALIGN, "the gated scan needs D >= 128, a multiple of 4, and 16-byte aligned rows");
   const int32_t kGatedTune = (8 << 8) | (vec << 16) | (1 << 24);
-  int rc = qssm_plan_scan_tuned(B, L, D, dtype, out_dtype, direction, align_elems, ckpt_stride, kGatedTune, plan);
-  if (rc == 0) plan->compute_dtype = compute_dtype;
-  if (rc != 0 || B == 0 || L == 0) return rc;
-  int g_log2 = plan->g_log2 > 6 ? 6 : (plan->g_log2 < 5 ? 5 : plan->g_log2);
-  if (g_log2 != plan->g_log2)
+  // The row width comes from a plan without a given spacing of saved states, so that the forward (which is handed
+  // the backward's tile length as that spacing) and the backward (which is handed it back) agree on it; the gated
+  // kernels exist for rows of 32 and 64 lanes.
+  int rc = qssm_plan_scan_tuned(B, L, D, dtype, out_dtype, direction, align_elems, 0, kGatedTune, plan);
+  if (rc != 0) return rc;
+  if (B == 0 || L == 0) {
+    rc = qssm_plan_scan_tuned(B, L, D, dtype, out_dtype, direction, align_elems, ckpt_stride, kGatedTune, plan);
+    if (rc == 0) plan->compute_dtype = compute_dtype;
+    return rc;
+  }
+  const int g_log2 = plan->g_log2 > 6 ? 6 : (plan->g_log2 < 5 ? 5 : plan->g_log2);
+  if (g_log2 != plan->g_log2 || ckpt_stride != 0)
     rc = qssm_plan_scan_tuned(B, L, D, dtype, out_dtype, direction, align_elems, ckpt_stride,
                               kGatedTune | (g_log2 + 1), plan);
   if (rc == 0 && plan->cluster > 2)   // same strips, more hand-overs, less LDS

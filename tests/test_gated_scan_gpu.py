@@ -160,6 +160,40 @@ def test_gated_scan_over_a_wide_tensor_past_4_gib(gpu):
     torch.cuda.empty_cache()
 
 
+@pytest.mark.timeout(600)
+def test_seeded_random_gated_shapes_match_the_oracle(gpu):
+    # A fixed-seed draw over (shape, projection storage, compute dtype): whatever geometry the planner picks for the
+    # gated launches (state widths from 128 up, clusters, partial strips, ragged last tiles) must meet the composed
+    # float64 oracle.  QSSM_RANDOM_GATED_CASES=n draws n cases instead of 60.
+    import os
+    n_cases = int(os.environ.get("QSSM_RANDOM_GATED_CASES", "60"))
+    rng = np.random.default_rng(20250911)
+    kinds = [(torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16), (torch.float32, torch.float16),
+             (torch.float32, torch.bfloat16), (torch.float32, torch.float32)]
+    for case in range(n_cases):
+        dtype, compute = kinds[case % len(kinds)]
+        unit = 8 if dtype != torch.float32 else 4                 # 16 bytes of a row
+        B = int(rng.integers(1, 4))
+        L = int(rng.choice([int(rng.integers(1, 100)), int(rng.integers(100, 1500)), int(rng.integers(1500, 5000))]))
+        S = max(128, unit * int(rng.choice([int(rng.integers(16, 40)), int(rng.integers(40, 130)), 32 * int(rng.integers(1, 5))])))
+        if B * L * S > 1_500_000:
+            L = max(1, 1_500_000 // (B * S))
+        shape = (B, L, S)
+        pre = _projections(shape, dtype, seed=3000 + case)
+        dy = torch.randn(shape, generator=torch.Generator().manual_seed(4000 + case)).to(dtype)
+        if case < 20 or case % 10 == 0:
+            print(f"case random gated {case} shape={shape} storage={dtype} compute={compute}", flush=True)
+        y_ref, g_ref = _oracle(pre, dy, compute)
+        y, grads = _run(pre, dy, gpu, dtype, compute_dtype=compute)
+        y_tol = {torch.float32: 2e-5, torch.float16: 1e-3, torch.bfloat16: 1e-2}[compute] if dtype == torch.float32 \
+            else TOL[dtype]
+        g_tol = (2e-5 if compute == torch.float32 else 1e-2) if dtype == torch.float32 else TOL[dtype]
+        assert_close(f"y (case {case})", y, y_ref, y_tol)
+        for name, got, want in zip(NAMES, grads, g_ref):
+            assert got.dtype == dtype
+            assert_close(f"{name} (case {case})", got, want, g_tol)
+
+
 def test_gated_forward_without_a_backward_equals_the_one_with(gpu):
     # no projection wants a gradient: the launch is planned with keep_tiles = 0; y is the same bit for bit
     pre = [t.to(gpu) for t in _projections((2, 900, 512), torch.bfloat16, seed=41)]

@@ -287,6 +287,33 @@ def test_plan_invariants_over_random_shapes(hip_lib):
         assert fwd.ckpt_stride == bwd.ckpt_stride == bwd.seg_len
 
 
+def test_gated_plans_of_both_directions_agree_on_the_saved_states(hip_lib):
+    # The gated forward is handed the gated backward's tile length as the spacing of its saved states, and the
+    # backward is handed it back: over a grid of shapes (very short sequences included, where the planner first
+    # widens the rows and the gated kernels then narrow them again) both plans must exist, keep that spacing and
+    # describe launches the gated kernels are built for.  (1, 6, 688) and (1, 7, 1008) failed to plan once.
+    from quick_ssm_amd import gated_scan
+    storage = ((torch.float16, (torch.float16,)), (torch.bfloat16, (torch.bfloat16,)),
+               (torch.float32, (torch.float16, torch.bfloat16, torch.float32)))
+    for dtype, computes in storage:
+        for compute in computes:
+            for B in (1, 2, 3, 16):
+                for L in (1, 2, 5, 6, 7, 8, 9, 16, 17, 31, 33, 64, 100, 257, 1000, 4096, 65536):
+                    for S in (128, 132, 136, 264, 512, 688, 1008, 1024, 4096):
+                        outs = (dtype, torch.float32) if dtype != torch.float32 else (torch.float32,)
+                        for out in outs:
+                            what = (B, L, S, dtype, compute, out)
+                            stride = gated_scan._plan(B, L, S, dtype, compute, dtype, _lib.QSSM_BACKWARD, 0).seg_len
+                            fwd = gated_scan._plan(B, L, S, dtype, compute, out, _lib.QSSM_FORWARD, stride)
+                            bwd = gated_scan._plan(B, L, S, dtype, compute, dtype, _lib.QSSM_BACKWARD, stride)
+                            assert bwd.seg_len == stride and fwd.seg_len % stride == 0, what
+                            assert fwd.ckpt_stride == bwd.ckpt_stride == stride, what
+                            for p in (fwd, bwd):
+                                assert p.threads == 256 and p.steps == 8 and p.g_log2 in (5, 6), what
+                                assert p.vec == 8 // torch.empty((), dtype=dtype).element_size() and p.cluster <= 2, what
+                                assert p.compute_dtype == gated_scan._CODES[compute], what
+
+
 def test_tile_index_arithmetic_over_random_shapes(hip_lib):
     # the same bounds model over a seeded sweep of small shapes, alignments, storage types and forced geometries
     import random
