@@ -362,7 +362,10 @@ int qssm_plan_scan_tuned(int32_t B, int32_t L, int32_t D, int32_t in_dtype, int3
     if ((ckpt_stride & (ckpt_stride - 1)) != 0 || ckpt_stride < 4)
       return fail(QSSM_EINVAL, "ckpt_stride=%d must be a power of two >= 4", ckpt_stride);
     if (direction == QSSM_FORWARD && ckpt_stride % steps != 0) steps = 4;
-    while (steps * (threads / g) < ckpt_stride && threads < kMaxThreads && vec > 1 && vec < 8) threads <<= 1;
+    // Longer tiles first through more lanes (as far as the kernels and the caller's choice go), then through
+    // narrower rows.
+    const int most_threads = (direction == QSSM_BACKWARD && vec == 4 && steps == 8) ? 512 : kMaxThreads;
+    while (steps * (threads / g) < ckpt_stride && !fixed_t && threads < most_threads && vec > 1 && vec < 8) threads <<= 1;
     while (steps * (threads / g) < ckpt_stride && g > 1) g >>= 1;
     if ((steps * (threads / g)) % ckpt_stride != 0)
       return fail(QSSM_EINVAL, "ckpt_stride=%d does not fit any tile length", ckpt_stride);

@@ -302,6 +302,60 @@ def test_ssm_layer_with_16_bit_parameters_uses_the_gated_scan_and_matches_the_se
         assert_close(f"grad {n}", g[n], g_ref[n].double().numpy(), tol)
 
 
+@pytest.mark.timeout(600)
+def test_seeded_random_layers_with_16_bit_parameters_match_the_sequential_path(gpu):
+    # A fixed-seed draw over layer sizes, batch, sequence length (down to one step) and 16-bit parameter types: the
+    # device layer (gated scan, fused or two-pass backward, wide or separate projections) against the same layer with
+    # the same parameter values in float64 on the product's sequential torch path on the CPU (a 16-bit run of that
+    # path is itself several roundings away from it).  QSSM_RANDOM_LAYER16_CASES=n draws n cases instead of 24.
+    import os
+    from quick_ssm_amd.layers import SSM
+
+    n_cases = int(os.environ.get("QSSM_RANDOM_LAYER16_CASES", "24"))
+    rng = np.random.default_rng(4242)
+    for case in range(n_cases):
+        dtype = (torch.bfloat16, torch.float16)[case % 2]
+        hidden = int(rng.choice([32, 64, 128, 256]))
+        mult = float(rng.choice([1.0, 2.0, 4.0]))
+        B = int(rng.integers(1, 3))
+        L = int(rng.choice([int(rng.integers(1, 12)), int(rng.integers(12, 120)), int(rng.integers(120, 260))]))
+        out32 = bool(rng.integers(0, 2))            # fp32 scan output: the two-pass backward
+        torch.manual_seed(700 + case)
+        layer = SSM(hidden_size=hidden, state_size_mult=mult, compute_dtype=dtype, dtype=dtype)
+        ref_layer = SSM(hidden_size=hidden, state_size_mult=mult, compute_dtype=torch.float64, dtype=torch.float64)
+        ref_layer.load_state_dict(layer.state_dict())           # the 16-bit values, exactly
+        layer = layer.to(gpu)
+        g = torch.Generator(device="cpu").manual_seed(800 + case)
+        xin = torch.randn(B, L, hidden, generator=g).to(dtype)
+        gout = torch.randn(B, L, hidden, generator=g).to(dtype)
+        kw = {"scan_out_dtype": torch.float32} if out32 else {}
+        print(f"case random 16-bit layer {case} B={B} L={L} hidden={hidden} state={int(hidden * mult)} {dtype} {kw}", flush=True)
+
+        def run(mod, inp, backend):
+            mod.zero_grad(set_to_none=True)
+            inp = inp.clone().requires_grad_(True)
+            out = mod(inp, backend=backend, **kw)
+            out.backward(gout.to(inp.device))
+            return (out.detach().cpu().float(), inp.grad.cpu().float(),
+                    {n: p.grad.cpu().float() for n, p in mod.named_parameters()})
+
+        def run_ref():
+            ref_layer.zero_grad(set_to_none=True)
+            inp = xin.double().requires_grad_(True)
+            out = ref_layer(inp, backend="torch", **({"scan_out_dtype": torch.float64} if out32 else {}))
+            out.backward(gout.double())
+            return out.detach(), inp.grad, {n: p.grad for n, p in ref_layer.named_parameters()}
+
+        y_ref, dx_ref, g_ref = run_ref()
+        y, dx, grads = run(layer, xin.to(gpu), "auto")
+        assert hip_scan.workspace_status() == 0
+        tol = 1e-2 if dtype == torch.float16 else 4e-2      # 16-bit parameters, activations and GEMM outputs
+        assert_close(f"layer out (case {case})", y, y_ref.numpy(), tol)
+        assert_close(f"layer dx (case {case})", dx, dx_ref.numpy(), tol)
+        for n in g_ref:
+            assert_close(f"grad {n} (case {case})", grads[n], g_ref[n].numpy(), tol)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 def test_batched_projection_gemm_equals_the_five_separate_ones(gpu, dtype, monkeypatch):
     # small layers stack the five projection weights into one batched GEMM; same values and gradients as five

@@ -308,6 +308,12 @@ def test_gated_plans_of_both_directions_agree_on_the_saved_states(hip_lib):
                             bwd = gated_scan._plan(B, L, S, dtype, compute, dtype, _lib.QSSM_BACKWARD, stride)
                             assert bwd.seg_len == stride and fwd.seg_len % stride == 0, what
                             assert fwd.ckpt_stride == bwd.ckpt_stride == stride, what
+                            # the two-pass backward (gate pass, then the plain backward over operands in the compute
+                            # dtype) reads the same saved states: the plain planner must take their spacing as well
+                            # ((2, 5, 1024) with fp32 dy failed to plan once)
+                            for align in (8, 4):
+                                plain = hip_scan.make_plan(B, L, S, compute, out, _lib.QSSM_BACKWARD, align, stride)
+                                assert plain.ckpt_stride == stride and plain.seg_len % stride == 0, (what, align)
                             for p in (fwd, bwd):
                                 assert p.threads == 256 and p.steps == 8 and p.g_log2 in (5, 6), what
                                 assert p.vec == 8 // torch.empty((), dtype=dtype).element_size() and p.cluster <= 2, what

@@ -354,6 +354,45 @@ def test_pieces_with_carried_state_equal_the_whole_scan(gpu, dtype, shape, cuts)
         assert_close(k + " (pieces vs whole)", got[k], whole[k].double().numpy(), TOL[dtype])
 
 
+def test_seeded_random_pieces_with_carried_state_match_the_oracle(gpu):
+    # A fixed-seed draw over (shape, storage, cut points, checkpoint on/off): a sequence scanned in pieces of random
+    # lengths (single steps included) with the state carried through autograd must give the whole sequence's y and
+    # gradients.  QSSM_RANDOM_PIECE_CASES=n draws n cases instead of 40.
+    n_cases = int(os.environ.get("QSSM_RANDOM_PIECE_CASES", "40"))
+    rng = np.random.default_rng(31337)
+    dtypes = (torch.float32, torch.float16, torch.bfloat16)
+    for case in range(n_cases):
+        dtype = dtypes[case % 3]
+        B = int(rng.integers(1, 4))
+        L = int(rng.choice([int(rng.integers(2, 40)), int(rng.integers(40, 700)), int(rng.integers(700, 2500))]))
+        D = int(rng.choice([int(rng.integers(1, 20)), 8 * int(rng.integers(1, 40)), 256 * int(rng.integers(1, 3))]))
+        n_cuts = int(rng.integers(1, 6))
+        cuts = sorted({0, L, *(int(v) for v in rng.integers(1, L, size=n_cuts))})
+        if rng.integers(0, 3) == 0 and L > 3:      # a run of single steps somewhere
+            t = int(rng.integers(1, L - 2))
+            cuts = sorted({*cuts, t, t + 1, t + 2})
+        checkpoint = bool(rng.integers(0, 2))
+        x, a, b, c, dy = make_inputs((B, L, D), dtype=dtype, seed=5000 + case)
+        if case < 12 or case % 10 == 0:
+            print(f"case random pieces {case} shape=({B}, {L}, {D}) {dtype} cuts={cuts} checkpoint={checkpoint}", flush=True)
+        ref = oracle_all(x, a, b, c, dy)
+        h64, _ = oracle.forward_f64(x, a, b, c)
+        leaves = [t.to(gpu).requires_grad_(True) for t in (x, a, b, c)]
+        state, ys = None, []
+        for k0, k1 in zip(cuts[:-1], cuts[1:]):
+            y, state = scan_chunk(*(t[:, k0:k1] for t in leaves), state, checkpoint=checkpoint)
+            ys.append(y)
+        assert_close(f"final state (case {case})", state.detach(), h64[:, -1], 1e-5)
+        y = torch.cat(ys, dim=1)
+        y.backward(dy.to(gpu))
+        assert hip_scan.workspace_status() == 0
+        got = {"y": y.detach().cpu()}
+        for k, t in zip(("dx", "da", "db", "dc"), leaves):
+            got[k] = t.grad.cpu()
+        for k in got:
+            assert_close(f"{k} (case {case})", got[k], ref[k], TOL[dtype])
+
+
 def test_token_by_token_generation_matches_scan(gpu):
     x, a, b, c, _ = make_inputs((2, 12, 520), dtype=torch.float16, seed=43)
     dev = [t.to(gpu) for t in (x, a, b, c)]
@@ -943,6 +982,39 @@ def test_ssm_layer_small_matches_oracle_composition(gpu):
     assert_close("layer dx", dx, ref_dx.numpy(), 1e-2)
     for n in ref_grads:
         assert_close(f"grad {n}", grads[n], ref_grads[n].numpy(), 1e-2)
+
+
+@pytest.mark.timeout(600)
+def test_seeded_random_layer_shapes_match_the_oracle_composition(gpu):
+    # A fixed-seed draw over layer sizes, batch, sequence length (down to a single step) and compute dtype, fp32
+    # parameters as the reference creates them: whichever route the layer takes (gated scan over one wide projection
+    # or over five, gate pass + plain scan for narrow states) must meet the float64 composition of the oracles.
+    # QSSM_RANDOM_LAYER_CASES=n draws n cases instead of 40.
+    from quick_ssm_amd.layers import SSM
+
+    n_cases = int(os.environ.get("QSSM_RANDOM_LAYER_CASES", "40"))
+    rng = np.random.default_rng(977)
+    computes = (torch.float16, torch.bfloat16, torch.float32)
+    for case in range(n_cases):
+        compute = computes[case % 3]
+        hidden = int(rng.choice([32, 64, 96, 128, 256]))
+        mult = float(rng.choice([1.0, 2.0, 4.0]))
+        B = int(rng.integers(1, 4))
+        L = int(rng.choice([int(rng.integers(1, 12)), int(rng.integers(12, 300)), int(rng.integers(300, 1200))]))
+        torch.manual_seed(500 + case)
+        layer = SSM(hidden_size=hidden, state_size_mult=mult, compute_dtype=compute, dtype=torch.float32).to(gpu)
+        g = torch.Generator(device="cpu").manual_seed(600 + case)
+        xin = torch.randn(B, L, hidden, generator=g)
+        gout = torch.randn(B, L, hidden, generator=g)
+        print(f"case random layer {case} B={B} L={L} hidden={hidden} state={int(hidden * mult)} compute={compute}", flush=True)
+        out, dx, grads = _run_layer(layer, xin.to(gpu), gout)
+        assert hip_scan.workspace_status() == 0
+        ref_out, ref_dx, ref_grads = _layer_oracle_f64(layer, xin, gout, "cpu")
+        tol = 1e-4 if compute == torch.float32 else 1e-2
+        assert_close(f"layer out (case {case})", out, ref_out.numpy(), tol)
+        assert_close(f"layer dx (case {case})", dx, ref_dx.numpy(), tol)
+        for n in ref_grads:
+            assert_close(f"grad {n} (case {case})", grads[n], ref_grads[n].numpy(), tol)
 
 
 @pytest.mark.timeout(900)
