@@ -1185,6 +1185,70 @@ def test_random_shapes_layouts_and_storage_against_oracle(gpu):
             assert_close(f"case {case} {name}", leaf.grad.cpu(), ref[name], tol_g)
 
 
+def test_seeded_random_operand_layouts_tiles_and_keywords(gpu):
+    # A fixed-seed draw in which every operand gets a layout of its own (dense, time-major memory, broadcast over the
+    # batch or over time through stride 0, a transposed last axis that needs a copy, a column block of a wider tensor,
+    # an offset that breaks 16-byte alignment) and scan() random keywords (block_l, checkpoint, tile_b, tile_d,
+    # out_dtype); gradients of broadcast operands come back summed by autograd.  QSSM_RANDOM_LAYOUT_CASES=n draws n
+    # cases instead of 60.
+    n_cases = int(os.environ.get("QSSM_RANDOM_LAYOUT_CASES", "60"))
+    rng = np.random.default_rng(8088)
+    pairs = [(torch.float32, torch.float32), (torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16),
+             (torch.float16, torch.float32), (torch.bfloat16, torch.float32)]
+    layouts = ("dense", "time_major", "bcast_batch", "bcast_time", "transposed", "columns", "offset")
+
+    def place(t, layout):
+        B, L, D = t.shape
+        t = t.to(gpu)
+        if layout == "time_major":                      # memory is [L, B, D]
+            return t.transpose(0, 1).contiguous().transpose(0, 1)
+        if layout == "bcast_batch":                     # one batch row, stride 0 over the batch
+            return t[:1].contiguous().expand(B, L, D)
+        if layout == "bcast_time":                      # one step, stride 0 over time
+            return t[:, :1].contiguous().expand(B, L, D)
+        if layout == "transposed":                      # memory is [B, D, L]: the last axis is not contiguous
+            return t.transpose(1, 2).contiguous().transpose(1, 2)
+        if layout == "columns":
+            wide = torch.zeros(B, L, D + 24, dtype=t.dtype, device=gpu)
+            wide[:, :, 16:16 + D] = t
+            return wide[:, :, 16:16 + D]
+        if layout == "offset":                          # starts one element into its allocation
+            flat = torch.zeros(B * L * D + 1, dtype=t.dtype, device=gpu)
+            flat[1:] = t.reshape(-1)
+            return flat[1:].view(B, L, D)
+        return t
+
+    for case in range(n_cases):
+        dtype, out_dtype = pairs[case % len(pairs)]
+        B = int(rng.integers(1, 4))
+        L = int(rng.choice([int(rng.integers(1, 40)), int(rng.integers(40, 400)), int(rng.integers(400, 1500))]))
+        D = int(rng.choice([int(rng.integers(1, 20)), 8 * int(rng.integers(1, 40)), 256 * int(rng.integers(1, 3))]))
+        lay = [str(rng.choice(layouts)) for _ in range(5)]
+        kw = {"block_l": int(rng.choice([1, 16, 100, 256, 1024])), "checkpoint": bool(rng.integers(0, 2)),
+              "tile_b": [None, 1, 2][int(rng.integers(0, 3))], "tile_d": [None, 8, 100, 256][int(rng.integers(0, 4))]}
+        x, a, b, c, dy = make_inputs((B, L, D), dtype=dtype, seed=7000 + case, out_dtype=out_dtype)
+        # what the device sees: a broadcast operand repeats its first batch row or first step
+        seen = []
+        for t, how in zip((x, a, b, c, dy), lay):
+            if how == "bcast_batch":
+                t = t[:1].expand(B, L, D).contiguous()
+            elif how == "bcast_time":
+                t = t[:, :1].expand(B, L, D).contiguous()
+            seen.append(t)
+        if case < 12 or case % 10 == 0:
+            print(f"case random layouts {case} shape=({B}, {L}, {D}) {dtype}->{out_dtype} {lay} {kw}", flush=True)
+        ref = oracle_all(*seen)
+        bases = [place(t, how) for t, how in zip((x, a, b, c), lay[:4])]
+        leaves = [t.detach().requires_grad_(True) for t in bases]
+        y = scan(*leaves, out_dtype=out_dtype, **kw)
+        y.backward(place(dy, lay[4]))
+        assert hip_scan.workspace_status() == 0
+        assert_close(f"y (case {case})", y.detach().cpu(), ref["y"], TOL[out_dtype])
+        for name, leaf in zip(("dx", "da", "db", "dc"), leaves):
+            assert leaf.grad.shape == (B, L, D), name
+            assert_close(f"{name} (case {case})", leaf.grad.cpu(), ref[name], TOL[dtype])
+
+
 def test_nan_in_an_input_stays_in_its_column_and_nothing_hangs(gpu):
     # one NaN in x: from that step on y, da and dc of that column are NaN (the state carries it), db only at that
     # step, dx nowhere; every other column is untouched, no tile waits for ever (the tags of the exchanged words
