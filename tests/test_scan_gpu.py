@@ -1249,6 +1249,51 @@ def test_seeded_random_operand_layouts_tiles_and_keywords(gpu):
             assert_close(f"{name} (case {case})", leaf.grad.cpu(), ref[name], TOL[dtype])
 
 
+def test_scans_from_several_threads_on_shared_and_private_streams(gpu):
+    # Six Python threads scan forward and backward at the same time, three on the default stream (one control block
+    # and workspace between them, launches numbered under the lock) and three on streams of their own; autograd adds
+    # its own thread for every backward.  Every result must be the bits the same call gives on a quiet device.
+    import threading
+
+    shapes = [((2, 900, 256), torch.bfloat16), ((1, 2100, 64), torch.float32), ((3, 300, 520), torch.float16)]
+    cases = []
+    for k, (shape, dtype) in enumerate(shapes):
+        ops = [t.to(gpu) for t in make_inputs(shape, dtype=dtype, seed=90 + k)]
+        leaves = [t.clone().requires_grad_(True) for t in ops[:4]]
+        y = scan(*leaves)
+        y.backward(ops[4])
+        cases.append((ops, y.detach().clone(), [t.grad.clone() for t in leaves]))
+    torch.cuda.synchronize()
+    errors = []
+
+    def work(idx, own_stream):
+        try:
+            ops, y_ref, g_ref = cases[idx % len(cases)]
+            stream = torch.cuda.Stream(device=gpu) if own_stream else torch.cuda.current_stream(gpu)
+            stream.wait_stream(torch.cuda.default_stream(gpu))
+            with torch.cuda.stream(stream):
+                for it in range(25):
+                    leaves = [t.clone().requires_grad_(True) for t in ops[:4]]
+                    y = scan(*leaves)
+                    y.backward(ops[4])
+                    stream.synchronize()
+                    if not torch.equal(y, y_ref) or any(not torch.equal(t.grad, g) for t, g in zip(leaves, g_ref)):
+                        errors.append(f"thread {idx} iteration {it}: results differ")
+                        return
+        except Exception as exc:  # noqa: BLE001 - reported by the main thread
+            errors.append(f"thread {idx}: {type(exc).__name__}: {exc}")
+
+    threads = [threading.Thread(target=work, args=(k, k >= 3)) for k in range(6)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=120)
+    assert not any(t.is_alive() for t in threads), "a worker thread did not finish"
+    torch.cuda.synchronize()
+    assert not errors, errors
+    assert hip_scan.workspace_status() == 0
+
+
 def test_nan_in_an_input_stays_in_its_column_and_nothing_hangs(gpu):
     # one NaN in x: from that step on y, da and dc of that column are NaN (the state carries it), db only at that
     # step, dx nowhere; every other column is untouched, no tile waits for ever (the tags of the exchanged words
