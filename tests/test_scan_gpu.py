@@ -701,6 +701,39 @@ def test_block_l_and_tiles_do_not_change_results(gpu, dtype):
         honor_tiles(old)
 
 
+def test_seeded_random_tiles_launched_one_by_one(gpu):
+    # With one launch per (tile_b, tile_d) tile, as the reference loops (quick_ssm/scan_interface.py:88-103): a
+    # fixed-seed draw over shapes, storage, odd tile sizes and checkpoint on/off; every tile is a strided view that
+    # may start off the 16-byte grid.  QSSM_RANDOM_TILE_CASES=n draws n cases instead of 30.
+    n_cases = int(os.environ.get("QSSM_RANDOM_TILE_CASES", "30"))
+    rng = np.random.default_rng(2718)
+    pairs = [(torch.float32, torch.float32), (torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16),
+             (torch.bfloat16, torch.float32)]
+    old = honor_tiles(True)
+    try:
+        for case in range(n_cases):
+            dtype, out_dtype = pairs[case % len(pairs)]
+            B = int(rng.integers(1, 6))
+            L = int(rng.choice([int(rng.integers(1, 50)), int(rng.integers(50, 900))]))
+            D = int(rng.choice([int(rng.integers(1, 30)), 8 * int(rng.integers(1, 40)), 256 * int(rng.integers(1, 3))]))
+            tile_b = [None, 1, 2, 3][int(rng.integers(0, 4))]
+            tile_d = [None, 1, 7, 8, 13, 100, 256][int(rng.integers(0, 7))]
+            checkpoint = bool(rng.integers(0, 2))
+            x, a, b, c, dy = make_inputs((B, L, D), dtype=dtype, seed=9000 + case, out_dtype=out_dtype)
+            if case < 10 or case % 10 == 0:
+                print(f"case random tiles {case} shape=({B}, {L}, {D}) {dtype}->{out_dtype} tile_b={tile_b} tile_d={tile_d} "
+                      f"checkpoint={checkpoint}", flush=True)
+            got = run_scan_with_grads(scan, x, a, b, c, dy, gpu, tile_b=tile_b, tile_d=tile_d, checkpoint=checkpoint,
+                                      out_dtype=out_dtype)
+            assert hip_scan.workspace_status() == 0
+            ref = oracle_all(x, a, b, c, dy)
+            assert_close(f"y (case {case})", got["y"], ref["y"], TOL[out_dtype])
+            for k in ("dx", "da", "db", "dc"):
+                assert_close(f"{k} (case {case})", got[k], ref[k], TOL[dtype])
+    finally:
+        honor_tiles(old)
+
+
 def test_launch_geometry_does_not_change_results_beyond_rounding(gpu):
     # every lanes-per-row / steps-per-lane geometry must agree with the oracle
     x, a, b, c, dy = make_inputs((2, 1100, 72), seed=8)
