@@ -72,6 +72,23 @@ def test_static_entry_point_equals_the_caller_buffer_one_twice_in_a_row(gpu, hip
     assert torch.equal(again[1][0], again[2][0]) and torch.equal(second[2][0], again[2][0])
 
 
+def test_static_entry_point_over_a_seeded_run_of_shapes(gpu, hip_lib):
+    # 25 calls in a row with changing shapes, storage and geometry, all through the one scratch array: each equals
+    # the caller-buffer entry point bit for bit (and meets the oracle, inside the helper)
+    import numpy as np
+
+    rng = np.random.default_rng(606)
+    dtypes = (torch.bfloat16, torch.float32, torch.float16)
+    for case in range(25):
+        dtype = dtypes[case % 3]
+        B = int(rng.integers(1, 4))
+        L = int(rng.choice([int(rng.integers(1, 100)), int(rng.integers(100, 1200)), int(rng.integers(1200, 4000))]))
+        D = 8 * int(rng.choice([int(rng.integers(1, 12)), int(rng.integers(12, 70)), 32 * int(rng.integers(1, 3))]))
+        print(f"case static {case} shape=({B}, {L}, {D}) {dtype}", flush=True)
+        plan, (y0, k0), (y1, k1) = _forward_both_ways(hip_lib, gpu, (B, L, D), dtype, seed=200 + case)
+        assert torch.equal(y0, y1) and torch.equal(k0, k1), (case, (B, L, D), dtype)
+
+
 def test_static_entry_point_refuses_what_does_not_fit(gpu, hip_lib):
     lib = hip_lib
     B, L, D = 64, 8192, 4096     # 8.6 G elements' worth of tiles: far more workspace than the array holds
