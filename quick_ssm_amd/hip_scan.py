@@ -344,10 +344,11 @@ _forward_keep = True
 
 
 def set_forward_keep(flag):
-    """Whether forwards planned from now on follow the planner's cache policy (`plan.keep_tiles`: the last tiles of
-    every chain load their operands with ordinary loads, for a backward that starts there; True), stream every
-    operand past the caches (False), or keep at most that many tiles per chain (an int).  Results are the same bit
-    for bit; only what a launch leaves in the caches differs.  Returns the old setting."""
+    """Whether forwards that save states for a backward (plain and gated) follow the planner's cache policy from now
+    on (`plan.keep_tiles`: the last tiles of every chain load their operands with ordinary loads, for a backward
+    that starts there; True), stream every operand past the caches (False), or keep at most that many tiles per
+    chain (an int).  Forwards that save nothing always stream.  Results are the same bit for bit; only what a launch
+    leaves in the caches differs.  Returns the old setting."""
     global _forward_keep
     old = _forward_keep
     _forward_keep = flag if isinstance(flag, bool) else max(0, int(flag))
